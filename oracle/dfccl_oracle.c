@@ -1,0 +1,469 @@
+/* CPU oracle for the DFCCL data path. Test infrastructure only; see dfccl_oracle.h
+ * for the reference lines every function follows and how each one is pinned. */
+#include "dfccl_oracle.h"
+
+#include <math.h>
+#include <pthread.h>
+#include <stdlib.h>
+#include <string.h>
+
+int orc_type_size(int dtype) {
+  switch (dtype) {
+    case ORC_I8: return 1;
+    case ORC_I32: return 4;
+    case ORC_F16: return 2;
+    case ORC_F32: return 4;
+    case ORC_BF16: return 2;
+    default: return 0;
+  }
+}
+
+/* ---------------------------------------------------------------- soft float */
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+uint16_t orc_f32_to_bf16(float f) {
+  uint32_t u = f2u(f);
+  if ((u & 0x7f800000u) == 0x7f800000u && (u & 0x007fffffu)) return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+  uint32_t lsb = (u >> 16) & 1u;
+  u += 0x7fffu + lsb; /* round to nearest, ties to even */
+  return (uint16_t)(u >> 16);
+}
+
+float orc_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+uint16_t orc_f32_to_f16(float f) {
+  uint32_t u = f2u(f);
+  uint32_t sign = (u >> 16) & 0x8000u;
+  uint32_t absu = u & 0x7fffffffu;
+  if (absu >= 0x7f800000u) { /* inf / nan */
+    if (absu > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((absu >> 13) & 0x3ffu));
+    return (uint16_t)(sign | 0x7c00u);
+  }
+  if (absu >= 0x477ff000u) { /* >= 65520 rounds to inf */
+    return (uint16_t)(sign | 0x7c00u);
+  }
+  if (absu < 0x38800000u) { /* below the smallest normal half 2^-14: subnormal result */
+    if (absu < 0x33000000u) { /* < 2^-25: rounds to zero (2^-25 itself ties to even = 0) */
+      return (uint16_t)sign;
+    }
+    /* value = mant * 2^(e-150); half subnormal unit is 2^-24 */
+    uint32_t e = absu >> 23;
+    uint32_t mant = (absu & 0x007fffffu) | 0x00800000u;
+    uint32_t shift = 126u - e; /* in [14, 24]: result = mant >> shift in units of 2^-24 */
+    uint32_t q = mant >> shift;
+    uint32_t rem = mant & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1u);
+    if (rem > half || (rem == half && (q & 1u))) q++;
+    return (uint16_t)(sign | q);
+  }
+  /* normal: rebias exponent 127 -> 15, round 13 dropped bits to nearest even */
+  uint32_t v = absu - 0x38000000u;
+  uint32_t lsb = (v >> 13) & 1u;
+  v += 0x0fffu + lsb;
+  return (uint16_t)(sign | (v >> 13));
+}
+
+float orc_f16_to_f32(uint16_t h) {
+  uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1fu;
+  uint32_t m = h & 0x3ffu;
+  if (e == 0) {
+    if (m == 0) return u2f(sign);
+    /* subnormal: m * 2^-24 */
+    float v = (float)m * 5.9604644775390625e-08f;
+    return u2f(f2u(v) | sign);
+  }
+  if (e == 31) return u2f(sign | 0x7f800000u | (m << 13));
+  return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+/* ------------------------------------------------------------- element ops */
+
+static inline float op_f32(int op, float a, float b) {
+  switch (op) {
+    case ORC_SUM: return a + b;
+    case ORC_PROD: return a * b;
+    case ORC_MAX: return fmaxf(a, b);
+    default: return fminf(a, b);
+  }
+}
+static inline int32_t op_i32(int op, int32_t a, int32_t b) {
+  switch (op) {
+    case ORC_SUM: return (int32_t)((uint32_t)a + (uint32_t)b);
+    case ORC_PROD: return (int32_t)((uint32_t)a * (uint32_t)b);
+    case ORC_MAX: return (a < b) ? b : a;
+    default: return (a < b) ? a : b;
+  }
+}
+static inline int8_t op_i8(int op, int8_t a, int8_t b) {
+  switch (op) {
+    case ORC_SUM: return (int8_t)(uint8_t)((uint8_t)a + (uint8_t)b);
+    case ORC_PROD: return (int8_t)(uint8_t)((unsigned)(uint8_t)a * (unsigned)(uint8_t)b);
+    case ORC_MAX: return (a > b) ? a : b;
+    default: return (a < b) ? a : b;
+  }
+}
+static inline uint16_t op_f16(int op, uint16_t a, uint16_t b) {
+  return orc_f32_to_f16(op_f32(op, orc_f16_to_f32(a), orc_f16_to_f32(b)));
+}
+static inline uint16_t op_bf16(int op, uint16_t a, uint16_t b) {
+  return orc_f32_to_bf16(op_f32(op, orc_bf16_to_f32(a), orc_bf16_to_f32(b)));
+}
+
+void orc_apply(int dtype, int op, const void* a, const void* b, void* out) {
+  switch (dtype) {
+    case ORC_I8: *(int8_t*)out = op_i8(op, *(const int8_t*)a, *(const int8_t*)b); break;
+    case ORC_I32: *(int32_t*)out = op_i32(op, *(const int32_t*)a, *(const int32_t*)b); break;
+    case ORC_F16: *(uint16_t*)out = op_f16(op, *(const uint16_t*)a, *(const uint16_t*)b); break;
+    case ORC_F32: *(float*)out = op_f32(op, *(const float*)a, *(const float*)b); break;
+    case ORC_BF16: *(uint16_t*)out = op_bf16(op, *(const uint16_t*)a, *(const uint16_t*)b); break;
+    default: break;
+  }
+}
+
+/* out[i] = op(a[i], b[i]) over a contiguous range; out may alias a or b. */
+#define RANGE_LOOP(T, FN)                                         \
+  do {                                                            \
+    const T* pa = (const T*)a; const T* pb = (const T*)b; T* po = (T*)out; \
+    switch (op) {                                                 \
+      case ORC_SUM: for (size_t i = 0; i < n; i++) po[i] = FN(ORC_SUM, pa[i], pb[i]); break;   \
+      case ORC_PROD: for (size_t i = 0; i < n; i++) po[i] = FN(ORC_PROD, pa[i], pb[i]); break; \
+      case ORC_MAX: for (size_t i = 0; i < n; i++) po[i] = FN(ORC_MAX, pa[i], pb[i]); break;   \
+      default: for (size_t i = 0; i < n; i++) po[i] = FN(ORC_MIN, pa[i], pb[i]); break;        \
+    }                                                             \
+  } while (0)
+
+static void apply_range(int dtype, int op, const void* a, const void* b, void* out, size_t n) {
+  switch (dtype) {
+    case ORC_I8: RANGE_LOOP(int8_t, op_i8); break;
+    case ORC_I32: RANGE_LOOP(int32_t, op_i32); break;
+    case ORC_F16: RANGE_LOOP(uint16_t, op_f16); break;
+    case ORC_F32: RANGE_LOOP(float, op_f32); break;
+    case ORC_BF16: RANGE_LOOP(uint16_t, op_bf16); break;
+    default: break;
+  }
+}
+
+/* ------------------------------------------------------------- reduce-copy */
+
+static void reduce_copy_range(int dtype, int op, int k, const void* const* srcs, void* dst, size_t begin, size_t n) {
+  size_t s = (size_t)orc_type_size(dtype);
+  char* d = (char*)dst + begin * s;
+  if (k == 1) {
+    memmove(d, (const char*)srcs[0] + begin * s, n * s);
+    return;
+  }
+  /* fold left to right; the first op reads src0 and src1, later ones the running value */
+  apply_range(dtype, op, (const char*)srcs[0] + begin * s, (const char*)srcs[1] + begin * s, d, n);
+  for (int j = 2; j < k; j++) apply_range(dtype, op, d, (const char*)srcs[j] + begin * s, d, n);
+}
+
+int orc_reduce_copy(int dtype, int op, int k, const void* const* srcs, void* dst, size_t n) {
+  if (orc_type_size(dtype) == 0 || k < 1 || op < 0 || op > 3) return -1;
+  reduce_copy_range(dtype, op, k, srcs, dst, 0, n);
+  return 0;
+}
+
+typedef struct {
+  int dtype, op, k;
+  const void* const* srcs;
+  void* dst;
+  size_t begin, n;
+} rc_job;
+
+static void* rc_thread(void* p) {
+  rc_job* j = (rc_job*)p;
+  reduce_copy_range(j->dtype, j->op, j->k, j->srcs, j->dst, j->begin, j->n);
+  return NULL;
+}
+
+int orc_reduce_copy_mt(int dtype, int op, int k, const void* const* srcs, void* dst, size_t n, int nthreads) {
+  if (orc_type_size(dtype) == 0 || k < 1 || op < 0 || op > 3) return -1;
+  if (nthreads <= 1) return orc_reduce_copy(dtype, op, k, srcs, dst, n);
+  if (nthreads > 256) nthreads = 256;
+  pthread_t th[256];
+  rc_job jobs[256];
+  size_t per = (n + (size_t)nthreads - 1) / (size_t)nthreads;
+  per = (per + 63) & ~(size_t)63;
+  int started = 0;
+  for (int t = 0; t < nthreads; t++) {
+    size_t b = (size_t)t * per;
+    if (b >= n) break;
+    size_t len = (n - b < per) ? n - b : per;
+    jobs[t] = (rc_job){dtype, op, k, srcs, dst, b, len};
+    if (pthread_create(&th[t], NULL, rc_thread, &jobs[t]) != 0) {
+      rc_thread(&jobs[t]);
+      th[t] = 0;
+      started = t + 1;
+      continue;
+    }
+    started = t + 1;
+  }
+  for (int t = 0; t < started; t++)
+    if (th[t]) pthread_join(th[t], NULL);
+  return 0;
+}
+
+/* ------------------------------------------------------------ ring schedule */
+
+static inline int64_t div_up(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline int64_t round_up(int64_t a, int64_t b) { return div_up(a, b) * b; }
+static inline int64_t min64(int64_t a, int64_t b) { return a < b ? a : b; }
+
+int64_t orc_real_chunk(int64_t chunk_elems, int64_t remaining, int64_t divisor, int64_t align_elems) {
+  int64_t r = min64(chunk_elems, div_up(remaining, divisor));
+  return round_up(r, align_elems);
+}
+
+static int geom_ok(const orc_geom* g) {
+  return g && g->n_ranks >= 1 && g->n_channels >= 1 && g->chunk_elems >= 1 && g->align_elems >= 1;
+}
+
+/* A message in flight on the link rank -> next rank: the data of one chunk. */
+typedef struct {
+  char* data;
+  int64_t nelem;
+} orc_msg;
+
+static void local_copy(int dtype, const void* src, void* dst, int64_t n) {
+  if (n > 0 && src != dst) memmove(dst, src, (size_t)n * (size_t)orc_type_size(dtype));
+}
+
+int orc_all_reduce(int dtype, int op, const orc_geom* g, int64_t count, const void* const* send, void* const* recv) {
+  if (!geom_ok(g) || orc_type_size(dtype) == 0) return -1;
+  const int n = g->n_ranks;
+  const size_t s = (size_t)orc_type_size(dtype);
+  if (n == 1) { local_copy(dtype, send[0], recv[0], count); return 0; }
+  const int64_t loop_size = (int64_t)g->n_channels * n * g->chunk_elems;
+  const int64_t max_chunk = round_up(g->chunk_elems, g->align_elems);
+  orc_msg* cur = calloc((size_t)n, sizeof(orc_msg));
+  orc_msg* prv = calloc((size_t)n, sizeof(orc_msg));
+  for (int r = 0; r < n; r++) {
+    cur[r].data = malloc((size_t)max_chunk * s);
+    prv[r].data = malloc((size_t)max_chunk * s);
+  }
+  for (int bid = 0; bid < g->n_channels; bid++) {
+    for (int64_t grid = 0; grid < count; grid += loop_size) {
+      const int64_t real = orc_real_chunk(g->chunk_elems, count - grid, (int64_t)g->n_channels * n, g->align_elems);
+      for (int step = 0; step < 2 * n - 1; step++) {
+        for (int r = 0; r < n; r++) {
+          const int prev = (r + n - 1) % n;
+          int chunk;
+          if (step == 0) chunk = (r + n - 1) % n;
+          else if (step <= n - 2) chunk = (r + n - (step + 1)) % n;
+          else if (step == n - 1) chunk = r;
+          else if (step <= 2 * n - 3) chunk = (r + n - (step - n + 1)) % n;
+          else chunk = (r + 1) % n;
+          const int64_t off = grid + (int64_t)bid * n * real + (int64_t)chunk * real;
+          int64_t nelem = min64(real, count - off);
+          if (nelem < 0) nelem = 0;
+          const char* in = (const char*)send[r] + (size_t)off * s;
+          char* out = (char*)recv[r] + (size_t)off * s;
+          if (step == 0) { /* send */
+            memcpy(cur[r].data, in, (size_t)nelem * s);
+          } else if (step <= n - 2) { /* recvReduceSend */
+            apply_range(dtype, op, in, prv[prev].data, cur[r].data, (size_t)nelem);
+          } else if (step == n - 1) { /* recvReduceCopySend */
+            apply_range(dtype, op, in, prv[prev].data, cur[r].data, (size_t)nelem);
+            memcpy(out, cur[r].data, (size_t)nelem * s);
+          } else if (step <= 2 * n - 3) { /* recvCopySend */
+            memcpy(cur[r].data, prv[prev].data, (size_t)nelem * s);
+            memcpy(out, cur[r].data, (size_t)nelem * s);
+          } else { /* recv */
+            memcpy(out, prv[prev].data, (size_t)nelem * s);
+          }
+          cur[r].nelem = nelem;
+        }
+        orc_msg* t = cur; cur = prv; prv = t;
+      }
+    }
+  }
+  for (int r = 0; r < n; r++) { free(cur[r].data); free(prv[r].data); }
+  free(cur); free(prv);
+  return 0;
+}
+
+int orc_all_reduce_owner(const orc_geom* g, int64_t count, int64_t i) {
+  const int n = g->n_ranks;
+  const int64_t loop_size = (int64_t)g->n_channels * n * g->chunk_elems;
+  const int64_t l = i / loop_size;
+  const int64_t grid = l * loop_size;
+  const int64_t real = orc_real_chunk(g->chunk_elems, count - grid, (int64_t)g->n_channels * n, g->align_elems);
+  const int64_t rel = i - grid;
+  const int64_t bid = rel / (n * real);
+  return (int)((rel - bid * n * real) / real);
+}
+
+int orc_reduce_scatter(int dtype, int op, const orc_geom* g, int64_t recvcount, const void* const* send,
+                       void* const* recv) {
+  if (!geom_ok(g) || orc_type_size(dtype) == 0) return -1;
+  const int n = g->n_ranks;
+  const size_t s = (size_t)orc_type_size(dtype);
+  if (n == 1) { local_copy(dtype, send[0], recv[0], recvcount); return 0; }
+  const int64_t loop_size = (int64_t)g->n_channels * g->chunk_elems;
+  const int64_t max_chunk = round_up(g->chunk_elems, g->align_elems);
+  orc_msg* cur = calloc((size_t)n, sizeof(orc_msg));
+  orc_msg* prv = calloc((size_t)n, sizeof(orc_msg));
+  for (int r = 0; r < n; r++) {
+    cur[r].data = malloc((size_t)max_chunk * s);
+    prv[r].data = malloc((size_t)max_chunk * s);
+  }
+  for (int bid = 0; bid < g->n_channels; bid++) {
+    for (int64_t grid = 0; grid < recvcount; grid += loop_size) {
+      const int64_t real = orc_real_chunk(g->chunk_elems, recvcount - grid, g->n_channels, g->align_elems);
+      const int64_t chunk_off = grid + (int64_t)bid * real;
+      int64_t nelem = min64(real, recvcount - chunk_off);
+      if (nelem < 0) nelem = 0;
+      for (int step = 0; step < n; step++) {
+        for (int r = 0; r < n; r++) {
+          const int prev = (r + n - 1) % n;
+          /* ringRanks[i] of rank r is (r + i) % n */
+          int dest;
+          if (step == 0) dest = (r + n - 1) % n;
+          else if (step <= n - 2) dest = (r + n - (step + 1)) % n;
+          else dest = r;
+          const int64_t off = chunk_off + (int64_t)dest * recvcount;
+          const char* in = (const char*)send[r] + (size_t)off * s;
+          if (step == 0) {
+            memcpy(cur[r].data, in, (size_t)nelem * s);
+          } else if (step <= n - 2) {
+            apply_range(dtype, op, in, prv[prev].data, cur[r].data, (size_t)nelem);
+          } else {
+            /* stage through the message buffer so an in-place recv buffer is safe */
+            apply_range(dtype, op, in, prv[prev].data, cur[r].data, (size_t)nelem);
+            memcpy((char*)recv[r] + (size_t)chunk_off * s, cur[r].data, (size_t)nelem * s);
+          }
+        }
+        orc_msg* t = cur; cur = prv; prv = t;
+      }
+    }
+  }
+  for (int r = 0; r < n; r++) { free(cur[r].data); free(prv[r].data); }
+  free(cur); free(prv);
+  return 0;
+}
+
+int orc_all_gather(int dtype, const orc_geom* g, int64_t sendcount, const void* const* send, void* const* recv) {
+  if (!geom_ok(g) || orc_type_size(dtype) == 0) return -1;
+  /* the reference runs all-gather on bytes: count *= sizeof(T), dtype = int8 */
+  const int n = g->n_ranks;
+  const int64_t size = sendcount * orc_type_size(dtype);
+  if (n == 1) { local_copy(ORC_I8, send[0], recv[0], size); return 0; }
+  const int64_t loop_size = (int64_t)g->n_channels * g->chunk_elems;
+  const int64_t max_chunk = round_up(g->chunk_elems, g->align_elems);
+  orc_msg* cur = calloc((size_t)n, sizeof(orc_msg));
+  orc_msg* prv = calloc((size_t)n, sizeof(orc_msg));
+  for (int r = 0; r < n; r++) {
+    cur[r].data = malloc((size_t)max_chunk);
+    prv[r].data = malloc((size_t)max_chunk);
+  }
+  for (int bid = 0; bid < g->n_channels; bid++) {
+    for (int64_t grid = 0; grid < size; grid += loop_size) {
+      const int64_t real = orc_real_chunk(g->chunk_elems, size - grid, g->n_channels, g->align_elems);
+      const int64_t chunk_off = grid + (int64_t)bid * real;
+      int64_t nelem = min64(real, size - chunk_off);
+      if (nelem < 0) nelem = 0;
+      for (int step = 0; step < n; step++) {
+        for (int r = 0; r < n; r++) {
+          const int prev = (r + n - 1) % n;
+          int dest;
+          if (step == 0) dest = r;
+          else if (step <= n - 2) dest = (r + n - step) % n;
+          else dest = (r + 1) % n;
+          const int64_t off = chunk_off + (int64_t)dest * size;
+          char* out = (char*)recv[r] + off;
+          if (step == 0) {
+            const char* in = (const char*)send[r] + chunk_off;
+            memcpy(cur[r].data, in, (size_t)nelem);
+            if (in != out) memmove(out, in, (size_t)nelem);
+          } else if (step <= n - 2) {
+            memcpy(cur[r].data, prv[prev].data, (size_t)nelem);
+            memcpy(out, cur[r].data, (size_t)nelem);
+          } else {
+            memcpy(out, prv[prev].data, (size_t)nelem);
+          }
+        }
+        orc_msg* t = cur; cur = prv; prv = t;
+      }
+    }
+  }
+  for (int r = 0; r < n; r++) { free(cur[r].data); free(prv[r].data); }
+  free(cur); free(prv);
+  return 0;
+}
+
+int orc_reduce(int dtype, int op, const orc_geom* g, int64_t count, int root, const void* const* send,
+               void* const* recv) {
+  if (!geom_ok(g) || orc_type_size(dtype) == 0) return -1;
+  const int n = g->n_ranks;
+  if (root < 0 || root >= n) return -1;
+  const size_t s = (size_t)orc_type_size(dtype);
+  if (n == 1) { local_copy(dtype, send[0], recv[0], count); return 0; }
+  const int64_t loop_size = (int64_t)g->n_channels * g->chunk_elems;
+  const int64_t max_chunk = round_up(g->chunk_elems, g->align_elems);
+  char* msg = malloc((size_t)max_chunk * s);
+  for (int bid = 0; bid < g->n_channels; bid++) {
+    for (int64_t grid = 0; grid < count; grid += loop_size) {
+      const int64_t real = orc_real_chunk(g->chunk_elems, count - grid, g->n_channels, g->align_elems);
+      const int64_t off = grid + (int64_t)bid * real;
+      int64_t nelem = min64(real, count - off);
+      if (nelem < 0) nelem = 0;
+      /* the chain starts at the rank whose predecessor is the root and ends at the root */
+      for (int k = 1; k <= n; k++) {
+        const int r = (root + k) % n;
+        const char* in = (const char*)send[r] + (size_t)off * s;
+        if (k == 1) {
+          memcpy(msg, in, (size_t)nelem * s); /* send */
+        } else if (k < n) {
+          apply_range(dtype, op, in, msg, msg, (size_t)nelem); /* recvReduceSend */
+        } else {
+          apply_range(dtype, op, in, msg, msg, (size_t)nelem); /* recvReduceCopy */
+          memcpy((char*)recv[r] + (size_t)off * s, msg, (size_t)nelem * s);
+        }
+      }
+    }
+  }
+  free(msg);
+  return 0;
+}
+
+int orc_broadcast(int dtype, const orc_geom* g, int64_t count, int root, const void* const* send, void* const* recv) {
+  if (!geom_ok(g) || orc_type_size(dtype) == 0) return -1;
+  const int n = g->n_ranks;
+  if (root < 0 || root >= n) return -1;
+  const int64_t size = count * orc_type_size(dtype);
+  if (n == 1) { local_copy(ORC_I8, send[0], recv[0], size); return 0; }
+  const int64_t loop_size = (int64_t)g->n_channels * g->chunk_elems;
+  for (int bid = 0; bid < g->n_channels; bid++) {
+    for (int64_t grid = 0; grid < size; grid += loop_size) {
+      const int64_t real = orc_real_chunk(g->chunk_elems, size - grid, g->n_channels, g->align_elems);
+      const int64_t off = grid + (int64_t)bid * real;
+      int64_t nelem = min64(real, size - off);
+      if (nelem <= 0) continue;
+      const char* src = (const char*)send[root] + off;
+      for (int k = 0; k < n; k++) {
+        const int r = (root + k) % n;
+        char* out = (char*)recv[r] + off;
+        if (out != src) memmove(out, src, (size_t)nelem);
+      }
+    }
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------ queues */
+
+uint64_t orc_cqe_encode(unsigned blk, unsigned cnt, unsigned coll_id) {
+  return ((uint64_t)(blk & 0xffu) << 56) | ((uint64_t)(cnt & 0xffffffu) << 32) | (uint64_t)coll_id;
+}
+
+void orc_cqe_decode(uint64_t v, unsigned* blk, unsigned* cnt, unsigned* coll_id) {
+  if (blk) *blk = (unsigned)(v >> 56);
+  if (cnt) *cnt = (unsigned)((v >> 32) & 0xffffffu);
+  if (coll_id) *coll_id = (unsigned)(v & 0xffffffffu);
+}
+
+int orc_sq_full(uint64_t head, uint64_t tail, uint64_t length) { return tail + 1 - head == length; }
+int orc_sq_empty(uint64_t frontier, uint64_t tail) { return frontier == tail; }
