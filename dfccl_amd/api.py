@@ -1,0 +1,182 @@
+"""Host-side mirror of the ofccl interface (src/nccl.h.in:202-378 in the
+reference) over the C ABI.  Method names and argument meaning follow the C
+entry points one to one; buffers are torch tensors that live on the GPU."""
+import ctypes
+import threading
+
+import torch
+
+from . import _lib
+from ._lib import CALLBACK, CollGeometry, Stats, UniqueId
+
+ncclSum, ncclProd, ncclMax, ncclMin = 0, 1, 2, 3
+ncclInt8, ncclInt32, ncclFloat16, ncclFloat32, ncclBfloat16 = 0, 2, 6, 7, 9
+
+DTYPE_OF = {torch.int8: ncclInt8, torch.int32: ncclInt32, torch.float16: ncclFloat16,
+            torch.float32: ncclFloat32, torch.bfloat16: ncclBfloat16}
+
+
+class NcclError(RuntimeError):
+    def __init__(self, code, what):
+        msg = _lib.load().ncclGetErrorString(code) if hasattr(_lib.load(), "ncclGetErrorString") else b""
+        super().__init__(f"{what}: ncclResult_t {code} ({(msg or b'').decode()})")
+        self.code = code
+
+
+def check(code, what="dfccl"):
+    if code != 0:
+        raise NcclError(code, what)
+
+
+def nccl_dtype(t):
+    try:
+        return DTYPE_OF[t.dtype]
+    except KeyError:
+        raise TypeError(f"dtype {t.dtype} is not on this path") from None
+
+
+def _dev_ptr(t):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("buffers must live on the GPU")
+    if not t.is_contiguous():
+        raise ValueError("buffers must be contiguous")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def reduce_copy(srcs, dst, op=ncclSum, chunk_bytes=0, stream=None):
+    """dst = srcs[0] (op) srcs[1] (op) ... folded left to right (dfcclReduceCopy). Asynchronous on `stream`
+    (default: torch's current stream)."""
+    lib = _lib.load()
+    n = dst.numel()
+    for s in srcs:
+        if s.dtype != dst.dtype or s.numel() != n:
+            raise ValueError("sources and destination must agree in dtype and length")
+    arr = (ctypes.c_void_p * len(srcs))(*[s.data_ptr() for s in srcs])
+    if stream is None:
+        stream = torch.cuda.current_stream(dst.device)
+    check(lib.dfcclReduceCopy(arr, len(srcs), _dev_ptr(dst), n, nccl_dtype(dst), op, chunk_bytes,
+                              ctypes.c_void_p(stream.cuda_stream)), "dfcclReduceCopy")
+
+
+class VirtualComm:
+    """One virtual rank's handle on a communicator (ncclCommInitRank)."""
+
+    def __init__(self, nranks, unique_id, rank):
+        self.handle = ctypes.c_void_p()
+        check(_lib.load().ncclCommInitRank(ctypes.byref(self.handle), nranks, unique_id, rank), "ncclCommInitRank")
+        self.nranks, self.rank = nranks, rank
+
+    @staticmethod
+    def unique_id():
+        uid = UniqueId()
+        check(_lib.load().ncclGetUniqueId(ctypes.byref(uid)), "ncclGetUniqueId")
+        return uid
+
+    @classmethod
+    def create_all(cls, nranks):
+        """The nranks handles of one fresh communicator, index = rank."""
+        uid = cls.unique_id()
+        return [cls(nranks, uid, r) for r in range(nranks)]
+
+    def destroy(self):
+        if self.handle:
+            check(_lib.load().ncclCommDestroy(self.handle), "ncclCommDestroy")
+            self.handle = ctypes.c_void_p()
+
+
+class RankCtx:
+    """ofcclRankCtx_t for one virtual rank: prepare*, finalize, run*, destroy."""
+
+    def __init__(self, rank):
+        self.lib = _lib.load()
+        self.rank = rank
+        self.handle = ctypes.c_void_p()
+        check(self.lib.ofcclInitRankCtx(ctypes.byref(self.handle), rank), "ofcclInitRankCtx")
+        self._keep = {}  # collId -> ctypes callback object, kept alive while in flight
+        self._lock = threading.Lock()
+
+    # -- prepare ------------------------------------------------------------
+    def prepare_all_reduce(self, count, dtype, op, comm, coll_id):
+        check(self.lib.ofcclPrepareAllReduce(count, dtype, op, comm.handle, coll_id, self.handle),
+              "ofcclPrepareAllReduce")
+
+    def prepare_reduce_scatter(self, recvcount, dtype, op, comm, coll_id):
+        check(self.lib.ofcclPrepareReduceScatter(recvcount, dtype, op, comm.handle, coll_id, self.handle),
+              "ofcclPrepareReduceScatter")
+
+    def prepare_all_gather(self, sendcount, dtype, comm, coll_id):
+        check(self.lib.ofcclPrepareAllGather(sendcount, dtype, comm.handle, coll_id, self.handle),
+              "ofcclPrepareAllGather")
+
+    def prepare_reduce(self, count, dtype, op, root, comm, coll_id):
+        check(self.lib.ofcclPrepareReduce(count, dtype, op, root, comm.handle, coll_id, self.handle),
+              "ofcclPrepareReduce")
+
+    def prepare_broadcast(self, count, dtype, root, comm, coll_id):
+        check(self.lib.ofcclPrepareBroadcast(count, dtype, root, comm.handle, coll_id, self.handle),
+              "ofcclPrepareBroadcast")
+
+    def prepare_bcast(self, count, dtype, root, comm, coll_id):
+        check(self.lib.ofcclPrepareBcast(count, dtype, root, comm.handle, coll_id, self.handle), "ofcclPrepareBcast")
+
+    def finalize(self):
+        check(self.lib.ofcclFinalizeRankCtx7StartHostThrds(self.handle), "ofcclFinalizeRankCtx7StartHostThrds")
+
+    def prepare_done(self):
+        check(self.lib.ofcclPrepareDone(self.handle), "ofcclPrepareDone")
+
+    # -- run ----------------------------------------------------------------
+    def _callback(self, coll_id, fn):
+        def tramp(cid, _args):
+            try:
+                if fn is not None:
+                    fn(cid)
+            except Exception:  # never let an exception cross the C boundary
+                import traceback
+                traceback.print_exc()
+            return 0
+        cb = CALLBACK(tramp)
+        with self._lock:
+            self._keep[coll_id] = cb
+        return cb
+
+    def _run(self, name, coll_id, fn, *bufs):
+        cb = self._callback(coll_id, fn)
+        check(getattr(self.lib, name)(*[_dev_ptr(b) for b in bufs], coll_id, cb, None, self.handle), name)
+
+    def run_all_reduce(self, send, recv, coll_id, callback=None):
+        self._run("ofcclRunAllReduce", coll_id, callback, send, recv)
+
+    def run_reduce_scatter(self, send, recv, coll_id, callback=None):
+        self._run("ofcclRunReduceScatter", coll_id, callback, send, recv)
+
+    def run_all_gather(self, send, recv, coll_id, callback=None):
+        self._run("ofcclRunAllGather", coll_id, callback, send, recv)
+
+    def run_reduce(self, send, recv, coll_id, callback=None):
+        self._run("ofcclRunReduce", coll_id, callback, send, recv)
+
+    def run_broadcast(self, send, recv, coll_id, callback=None):
+        self._run("ofcclRunBroadcast", coll_id, callback, send, recv)
+
+    def run_bcast(self, buf, coll_id, callback=None):
+        self._run("ofcclRunBcast", coll_id, callback, buf)
+
+    # -- introspection --------------------------------------------------------
+    def stats(self):
+        s = Stats()
+        check(self.lib.dfcclGetStats(self.handle, ctypes.byref(s)), "dfcclGetStats")
+        return {n: getattr(s, n) for n, _ in Stats._fields_}
+
+    def geometry(self, coll_id):
+        g = CollGeometry()
+        check(self.lib.dfcclGetCollGeometry(self.handle, coll_id, ctypes.byref(g)), "dfcclGetCollGeometry")
+        return g
+
+    def destroy(self):
+        if self.handle:
+            check(self.lib.ofcclDestroy(self.handle), "ofcclDestroy")
+            self.handle = ctypes.c_void_p()
+            self._keep.clear()

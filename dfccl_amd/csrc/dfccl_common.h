@@ -1,0 +1,162 @@
+// Data structures shared by the host runtime and the daemon kernel.
+//
+// Where each one lives:
+//   host-coherent (fine-grained, hipHostMalloc): submission ring, its head,
+//     completion ring, control word, per-workgroup exit flags and counters;
+//   HBM: mirror of the submission ring, per-collective plans, per-(workgroup,
+//     collective) contexts, FIFO slots and their head/tail flags, saved
+//     workgroup state.
+// They take the place of the reference's SQE/SQ/CQE/CQ, StaticCollCtx,
+// DynamicCollCtx, BlkStatus and ncclConnInfo (src/include/collectives_ofccl.h:
+// 129-157,171-183,328-355; src/include/devcomm.h:81-97).
+#pragma once
+
+#include <stdint.h>
+
+#include "ring_schedule.h"
+
+namespace dfccl {
+
+constexpr int kMaxColls = 2000;      // collIds and collectives per rank context (MAX_LENGTH)
+constexpr int kSqCapacity = 2000;    // submissions that may be outstanding per rank (QLen)
+constexpr int kSqRing = 2048;        // ring size, a power of two >= kSqCapacity + 1
+constexpr int kCqRing = 4096;        // completions can never outnumber kMaxColls in flight
+constexpr int kWgThreads = 512;      // daemon workgroup: 8 wave64
+constexpr int kMaxRankSlots = 16;    // virtual ranks one device daemon serves
+constexpr int kMaxChannels = 64;     // workgroups per virtual rank
+constexpr int kAlignBytes = 1024;    // chunk rounding unit: one wave's 128-bit access
+constexpr int kSqeWords = 4;         // 64-bit words per submission entry
+constexpr int kSqesPerPoll = 15;     // entries one wave fetches per poll (lane 60 reads the control word)
+constexpr uint64_t kPtrMask = 0x0000ffffffffffffull;  // device pointers fit 48 bits
+constexpr uint32_t kInvalidTask = 0xffffu;
+
+// Submission entry in host-coherent memory: four 64-bit words, each tagged in
+// its top 16 bits with (ticket + 1) & 0xffff so that a word can be validated on
+// its own (the device reads the words of an entry with independent loads).
+//   word 0: sendbuff | tag     word 1: recvbuff | tag
+//   word 2: collIndex (32) | flags (16) | tag     word 3: tag only
+constexpr uint32_t kSqeFlagQuit = 1u;
+
+DFCCL_HD uint64_t sqeTag(uint64_t ticket) { return ((ticket + 1) & 0xffffull) << 48; }
+
+// Control word the host writes, read by each rank's leader workgroup.
+constexpr uint32_t kCtrlQuitRequest = 1u;  // save state and leave (the host will relaunch)
+constexpr uint32_t kCtrlAbort = 2u;        // leave at once, state is abandoned
+
+// How a workgroup left the kernel (written to its host-coherent exit word as
+// epoch << 4 | kind, epoch = launch number).
+enum ExitKind : uint32_t { kExitNone = 0, kExitVoluntary = 1, kExitFinal = 2, kExitAbort = 3, kExitUnused = 4 };
+
+// Mirror of one submission in HBM, written by the rank's leader workgroup.
+struct alignas(32) DevSqe {
+  uint64_t sendbuff;
+  uint64_t recvbuff;
+  uint32_t coll;   // dense collective index of this rank context
+  uint32_t flags;
+  uint64_t ticket;
+};
+
+// Flow-control words of one FIFO (one link, one channel). tail counts slices the
+// sender has published, head slices the receiver has released.
+struct alignas(128) ConnFlags {
+  uint64_t tail;
+  uint64_t pad0[7];
+  uint64_t head;
+  uint64_t pad1[7];
+};
+
+// Immutable plan of one collective on one rank (HBM, written at finalize).
+struct alignas(16) CollPlan {
+  int32_t kind, dtype, op, root;
+  int32_t nRanks, rank, nChannels, collId;
+  int64_t count;        // elements of the run dtype (bytes for all-gather / broadcast)
+  int64_t chunkElems;   // nominal chunk
+  int64_t alignElems;
+  int64_t sliceElems;   // nominal slice = FIFO slot capacity in elements
+  int32_t slicesPerChunk, fifoSlots;
+  int32_t elemSize, pad;
+  int64_t slotBytes;
+  int64_t fifoChanStride;  // bytes between two channels' FIFOs of one link
+  char* sendFifo;          // link rank -> next, channel 0
+  char* recvFifo;          // link prev -> rank, channel 0
+  ConnFlags* sendFlags;    // indexed by channel
+  ConnFlags* recvFlags;
+  uint64_t* doneCounter;   // workgroups that finished an instance, monotonic
+};
+
+// Resumable position of one collective on one workgroup (HBM). This is the
+// context a preemption saves and a resume restores.
+struct alignas(64) DynCtx {
+  uint64_t sendbuff;
+  uint64_t recvbuff;
+  int64_t gridOffset;   // loop the workgroup is in
+  int32_t step;         // ring step inside the loop
+  int32_t slice;        // slice inside the step's chunk
+  uint64_t sendStep;    // slices ever sent on the send link (persists across instances)
+  uint64_t recvStep;    // slices ever received on the receive link
+  int32_t tryCnt;       // scheduler visits since the instance started
+  int32_t active;
+  uint64_t pad;
+};
+
+// Counters of one workgroup, in host-coherent memory so the host can read them
+// while the daemon runs.
+struct alignas(64) WgStats {
+  uint64_t sqesRead, cqesWritten, ctxSaves, ctxLoads, voluntaryQuits, forcedQuits, slicesMoved, spins;
+};
+
+// Scheduler state a workgroup saves when it leaves voluntarily and restores at
+// the next launch (HBM).
+struct WgSaved {
+  uint64_t frontier;      // next mirror-ring ticket to read
+  uint64_t hostFrontier;  // leader only: next host-ring ticket to read
+  int32_t numActive;
+  int32_t finalQuit;
+  uint16_t taskq[kMaxColls];
+};
+
+// Everything the kernel needs about one virtual rank.
+struct RankDev {
+  int32_t active;
+  int32_t nChannels;   // workgroups this rank uses (<= grid channels)
+  int32_t nColls;
+  int32_t rank;
+  // host-coherent
+  uint64_t* sq;        // kSqRing * kSqeWords words
+  uint64_t* sqHead;    // written by the leader: every workgroup has consumed tickets < *sqHead
+  uint64_t* cq;        // kCqRing entries
+  uint32_t* ctrl;      // control word (shared by all ranks of the daemon)
+  uint32_t* wgExit;    // [kMaxChannels]
+  WgStats* stats;      // [kMaxChannels]
+  // HBM
+  DevSqe* mirror;      // kSqRing entries
+  uint64_t* mirrorTail;
+  uint64_t* wgFrontier;  // [kMaxChannels]
+  uint64_t* cqTicket;
+  CollPlan* plans;     // [nColls]
+  DynCtx* dyn;         // [kMaxChannels][nColls]
+  WgSaved* saved;      // [kMaxChannels]
+};
+
+// Scheduling knobs; names and defaults are the reference's environment
+// variables (src/enqueue_ofccl.cc:763,1287-1297).
+struct Knobs {
+  int64_t baseCtxSwitchThreshold;   // BASE_CTX_SWITCH_THRESHOLD, default 80
+  int64_t numTryTaskqHead;          // NUM_TRY_TASKQ_HEAD, default 5
+  int64_t recvSuccessFactor;        // RECV_SUCCESS_FACTOR, default 5
+  int64_t tolerantUnprogressedCnt;  // TOLERANT_UNPROGRESSED_CNT, default 500000
+  int64_t forceQuitEvery;           // DFCCL_FORCE_QUIT_EVERY: preempt after this many slices (0 = off)
+  int64_t maxLifetimeTicks;         // DFCCL_DAEMON_MAX_MS in 100 MHz ticks (0 = unlimited)
+};
+
+struct DaemonArgs {
+  RankDev ranks[kMaxRankSlots];
+  Knobs knobs;
+  int32_t nSlots;
+  int32_t channelsPerRank;
+  uint32_t epoch;
+  uint32_t pad;
+  uint32_t* devFlags;  // HBM: [0] quit request, [1] abort (set by leaders from the control word)
+};
+
+}  // namespace dfccl

@@ -1,0 +1,901 @@
+// Host runtime of the DFCCL data path: rank contexts, virtual communicators,
+// submission / completion queues, the per-device daemon launcher ("observer")
+// and the per-rank completion poller.  Mirrors src/enqueue_ofccl.cc of the
+// reference (rank context :751, prepare :773, finalize :1285, sqWrite :616,
+// cqRead :697, poller :908, observer :967, destroy :1582) and the shims in
+// src/collectives_ofccl/ofccl_*.cc, over the HIP runtime.
+//
+// One daemon kernel serves all rank contexts of a device (they are virtual
+// ranks sharing one GPU), so the daemon object is per device and rank contexts
+// attach to one of its slots.
+#include <hip/hip_runtime.h>
+#include <immintrin.h>
+#include <sched.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <chrono>
+#include <condition_variable>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <thread>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/ofccl.h"
+#include "dfccl_common.h"
+
+#define DFCCL_API extern "C" __attribute__((visibility("default")))
+
+extern "C" hipError_t dfcclLaunchDaemon(const dfccl::DaemonArgs* devArgs, int nSlots, int channelsPerRank,
+                                        hipStream_t stream);
+
+namespace dfccl {
+
+#define HIPCHECK(call)                                                                                  \
+  do {                                                                                                  \
+    hipError_t e_ = (call);                                                                             \
+    if (e_ != hipSuccess) {                                                                             \
+      fprintf(stderr, "dfccl: %s failed: %s (%s:%d)\n", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
+      return ncclUnhandledCudaError;                                                                    \
+    }                                                                                                   \
+  } while (0)
+
+static int64_t envInt(const char* name, int64_t dflt) {
+  const char* v = getenv(name);
+  if (v == nullptr || *v == 0) return dflt;
+  char* end = nullptr;
+  long long x = strtoll(v, &end, 10);
+  return (end == v) ? dflt : (int64_t)x;
+}
+
+static int typeSizeOf(int dt) {
+  switch (dt) {
+    case ncclInt8: case ncclUint8: return 1;
+    case ncclFloat16: case ncclBfloat16: return 2;
+    case ncclInt32: case ncclUint32: case ncclFloat32: return 4;
+    case ncclInt64: case ncclUint64: case ncclFloat64: return 8;
+    default: return 0;
+  }
+}
+
+// dtypes the reduce kernels implement; copies (all-gather, broadcast) take any type
+static bool reduceDtypeSupported(int dt) {
+  return dt == ncclInt8 || dt == ncclInt32 || dt == ncclFloat16 || dt == ncclFloat32 || dt == ncclBfloat16;
+}
+
+// ------------------------------------------------------------------ communicators
+
+struct CommGroup {
+  uint64_t id = 0;
+  int nRanks = 0;
+  int device = 0;
+  std::mutex mu;
+  int handles = 0;
+  // the collective this communicator serves, fixed by the first Prepare
+  bool planned = false;
+  int kind = 0, dtypeUser = 0, op = 0, root = 0;
+  size_t countUser = 0;
+  // derived plan
+  int dtype = 0, elemSize = 1, nChannels = 1, slicesPerChunk = 1, fifoSlots = 1;
+  int64_t count = 0, chunkElems = 0, alignElems = 0, sliceElems = 0, slotBytes = 0, chanStride = 0;
+  // device memory: [nRanks links][nChannels] FIFOs and flags; link r goes from rank r to rank (r+1)%n
+  char* fifo = nullptr;
+  ConnFlags* flags = nullptr;
+};
+
+}  // namespace dfccl
+
+struct ncclComm {
+  dfccl::CommGroup* group;
+  int rank;
+  bool registered;
+};
+
+namespace dfccl {
+
+static std::mutex gCommMu;
+static std::unordered_map<uint64_t, CommGroup*> gGroups;
+static std::atomic<uint64_t> gNextCommId{1};
+
+struct Daemon;
+
+struct CollReg {
+  int collId;
+  ncclComm* comm;
+};
+
+}  // namespace dfccl
+
+struct ofcclRankCtx {
+  int rank = 0;
+  int device = 0;
+  std::vector<dfccl::CollReg> colls;
+  int16_t collIndex[dfccl::kMaxColls];
+  bool finalized = false;
+  dfccl::Daemon* daemon = nullptr;
+  int slot = -1;
+  int nChannels = 1;
+  dfccl::RankDev dev{};
+  uint64_t* doneCounters = nullptr;
+  // submission side
+  std::mutex sqMu;
+  uint64_t sqTail = 0;
+  // completion side
+  uint64_t cqRead = 0;
+  CallbackFunc callbacks[dfccl::kMaxColls];
+  void* cbArgs[dfccl::kMaxColls];
+  std::atomic<int> inflight[dfccl::kMaxColls];
+  std::atomic<uint64_t> submitted{0}, completed{0};
+  std::thread poller;
+  std::atomic<bool> stopPoller{false};
+  std::mutex pollMu;
+  std::condition_variable pollCv;
+};
+
+namespace dfccl {
+
+// ------------------------------------------------------------------------ daemon
+
+struct Daemon {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  hipEvent_t doneEv = nullptr;
+  std::mutex mu;
+  std::condition_variable cv;
+  ofcclRankCtx* slots[kMaxRankSlots] = {};
+  int nActive = 0;
+  bool running = false;
+  bool shutdown = false;
+  bool launchRequested = false;
+  bool failed = false;
+  uint32_t epoch = 0;
+  uint64_t launches = 0;
+  uint32_t* ctrl = nullptr;      // host-coherent
+  uint32_t* devFlags = nullptr;  // HBM
+  DaemonArgs* devArgs = nullptr; // HBM
+  DaemonArgs hostArgs{};
+  Knobs knobs{};
+  std::thread observer;
+  std::vector<void*> garbageDev, garbageHost;
+
+  bool wantLaunch() const {
+    if (launchRequested) return true;
+    for (int s = 0; s < kMaxRankSlots; s++) {
+      const ofcclRankCtx* c = slots[s];
+      if (c && c->submitted.load(std::memory_order_acquire) > c->completed.load(std::memory_order_acquire)) return true;
+    }
+    return false;
+  }
+
+  void collectGarbage() {  // only while the kernel is not running: hipFree waits for the device
+    for (void* p : garbageDev) (void)hipFree(p);
+    for (void* p : garbageHost) (void)hipHostFree(p);
+    garbageDev.clear();
+    garbageHost.clear();
+  }
+
+  void readKnobs() {
+    knobs.baseCtxSwitchThreshold = envInt("BASE_CTX_SWITCH_THRESHOLD", 80);
+    knobs.numTryTaskqHead = envInt("NUM_TRY_TASKQ_HEAD", 5);
+    knobs.recvSuccessFactor = envInt("RECV_SUCCESS_FACTOR", 5);
+    knobs.tolerantUnprogressedCnt = envInt("TOLERANT_UNPROGRESSED_CNT", 500000);
+    knobs.forceQuitEvery = envInt("DFCCL_FORCE_QUIT_EVERY", 0);
+    knobs.maxLifetimeTicks = envInt("DFCCL_DAEMON_MAX_MS", 0) * 100000;  // wall_clock64 runs at 100 MHz
+    if (knobs.numTryTaskqHead < 1) knobs.numTryTaskqHead = 1;
+    if (knobs.tolerantUnprogressedCnt < 1) knobs.tolerantUnprogressedCnt = 1;
+  }
+
+  // Launches the kernel for the current set of slots. Caller holds mu; the kernel is not running.
+  bool launchLocked() {
+    int nSlots = 0, chans = 1;
+    memset(&hostArgs, 0, sizeof(hostArgs));
+    for (int s = 0; s < kMaxRankSlots; s++) {
+      if (slots[s] == nullptr) continue;
+      hostArgs.ranks[s] = slots[s]->dev;
+      hostArgs.ranks[s].active = 1;
+      nSlots = s + 1;
+      if (slots[s]->nChannels > chans) chans = slots[s]->nChannels;
+    }
+    if (nSlots == 0) return false;
+    // a multiple of 8 channels keeps channel c of every rank on XCD c % 8
+    if (chans > 1) chans = (chans + 7) & ~7;
+    epoch++;
+    hostArgs.knobs = knobs;
+    hostArgs.nSlots = nSlots;
+    hostArgs.channelsPerRank = chans;
+    hostArgs.epoch = epoch;
+    hostArgs.devFlags = devFlags;
+    __atomic_store_n(ctrl, 0u, __ATOMIC_RELEASE);
+    if (hipMemcpy(devArgs, &hostArgs, sizeof(hostArgs), hipMemcpyHostToDevice) != hipSuccess) return false;
+    if (hipMemset(devFlags, 0, 64) != hipSuccess) return false;
+    if (dfcclLaunchDaemon(devArgs, nSlots, chans, stream) != hipSuccess) return false;
+    if (hipEventRecord(doneEv, stream) != hipSuccess) return false;
+    running = true;
+    launches++;
+    return true;
+  }
+
+  // (Re)launches the kernel whenever work is outstanding and it is not running
+  // (startKernel7SqObserver, src/enqueue_ofccl.cc:967-985).
+  void observerLoop() {
+    (void)hipSetDevice(device);
+    std::unique_lock<std::mutex> lk(mu);
+    for (;;) {
+      cv.wait(lk, [&] { return shutdown || (!failed && wantLaunch()); });
+      if (shutdown) break;
+      launchRequested = false;
+      if (!launchLocked()) {
+        fprintf(stderr, "dfccl: daemon launch failed on device %d: %s\n", device, hipGetErrorString(hipGetLastError()));
+        failed = true;
+        cv.notify_all();
+        continue;
+      }
+      cv.notify_all();
+      lk.unlock();
+      hipError_t e = hipEventSynchronize(doneEv);
+      lk.lock();
+      running = false;
+      if (e != hipSuccess) {
+        fprintf(stderr, "dfccl: daemon kernel ended with %s\n", hipGetErrorString(e));
+        failed = true;
+      }
+      collectGarbage();
+      cv.notify_all();
+    }
+  }
+
+  // Asks a running kernel to save its state and leave; returns once it has. Caller holds lk.
+  void quiesceLocked(std::unique_lock<std::mutex>& lk) {
+    if (!running) return;
+    __atomic_store_n(ctrl, kCtrlQuitRequest, __ATOMIC_RELEASE);
+    if (!cv.wait_for(lk, std::chrono::seconds(20), [&] { return !running; })) {
+      fprintf(stderr, "dfccl: daemon did not leave on request, aborting it\n");
+      __atomic_store_n(ctrl, kCtrlAbort, __ATOMIC_RELEASE);
+      cv.wait_for(lk, std::chrono::seconds(20), [&] { return !running; });
+    }
+  }
+};
+
+static std::mutex gDaemonMu;
+static std::map<int, Daemon*> gDaemons;
+static bool gAtexitRegistered = false;
+
+static void abortAllDaemonsAtExit() {
+  std::lock_guard<std::mutex> g(gDaemonMu);
+  for (auto& kv : gDaemons) {
+    Daemon* d = kv.second;
+    std::unique_lock<std::mutex> lk(d->mu);
+    if (d->running) {
+      __atomic_store_n(d->ctrl, kCtrlAbort, __ATOMIC_RELEASE);
+      d->cv.wait_for(lk, std::chrono::seconds(5), [&] { return !d->running; });
+    }
+  }
+}
+
+static ncclResult_t getDaemon(int device, Daemon** out) {
+  std::lock_guard<std::mutex> g(gDaemonMu);
+  auto it = gDaemons.find(device);
+  if (it != gDaemons.end()) {
+    *out = it->second;
+    return ncclSuccess;
+  }
+  Daemon* d = new Daemon();
+  d->device = device;
+  HIPCHECK(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
+  HIPCHECK(hipEventCreateWithFlags(&d->doneEv, hipEventBlockingSync | hipEventDisableTiming));
+  HIPCHECK(hipHostMalloc((void**)&d->ctrl, 64, hipHostMallocCoherent | hipHostMallocMapped));
+  *d->ctrl = 0;
+  HIPCHECK(hipMalloc((void**)&d->devFlags, 64));
+  HIPCHECK(hipMemset(d->devFlags, 0, 64));
+  HIPCHECK(hipMalloc((void**)&d->devArgs, sizeof(DaemonArgs)));
+  d->readKnobs();
+  d->observer = std::thread([d] { d->observerLoop(); });
+  gDaemons[device] = d;
+  if (!gAtexitRegistered) {
+    atexit(abortAllDaemonsAtExit);
+    gAtexitRegistered = true;
+  }
+  *out = d;
+  return ncclSuccess;
+}
+
+// Called with no rank attached any more: stops the observer and frees the daemon.
+static void destroyDaemon(Daemon* d) {
+  {
+    std::lock_guard<std::mutex> g(gDaemonMu);
+    gDaemons.erase(d->device);
+  }
+  {
+    std::unique_lock<std::mutex> lk(d->mu);
+    if (d->running) {
+      // every rank has left; whatever is still resident only has to notice
+      if (!d->cv.wait_for(lk, std::chrono::seconds(10), [&] { return !d->running; })) {
+        __atomic_store_n(d->ctrl, kCtrlAbort, __ATOMIC_RELEASE);
+        d->cv.wait_for(lk, std::chrono::seconds(10), [&] { return !d->running; });
+      }
+    }
+    d->shutdown = true;
+    d->cv.notify_all();
+  }
+  if (d->observer.joinable()) d->observer.join();
+  d->collectGarbage();
+  (void)hipFree(d->devArgs);
+  (void)hipFree(d->devFlags);
+  (void)hipHostFree(d->ctrl);
+  (void)hipEventDestroy(d->doneEv);
+  (void)hipStreamDestroy(d->stream);
+  delete d;
+}
+
+// ------------------------------------------------------------------------ planning
+
+// Fixes the chunk geometry of the collective a communicator serves
+// (ofcclComputeColl / ofcclGetAlgoInfo, src/enqueue_ofccl.cc:85-283: ring, one
+// protocol, channel count shrunk for small messages).
+static void planGroup(CommGroup* g) {
+  const int es = typeSizeOf(g->dtypeUser);
+  int64_t nBytes = (int64_t)g->countUser * es;
+  if (g->kind == kAllGather || g->kind == kBroadcast) {  // run as bytes (src/misc/argcheck.cc:53-57)
+    g->dtype = ncclInt8;
+    g->elemSize = 1;
+    g->count = nBytes;
+  } else {
+    g->dtype = g->dtypeUser;
+    g->elemSize = es;
+    g->count = (int64_t)g->countUser;
+  }
+  if (g->kind == kAllGather || g->kind == kReduceScatter) nBytes *= g->nRanks;
+  int64_t buff = envInt("NCCL_BUFFSIZE", 1 << 20);
+  if (buff < (64 << 10)) buff = 64 << 10;
+  buff = (buff / (8 * kAlignBytes)) * (8 * kAlignBytes);
+  const int64_t stepBytes = buff / 8;  // NCCL_STEPS = 8
+  int64_t chunkBytes, sliceBytes;
+  if (g->kind == kReduce || g->kind == kBroadcast) {  // CHUNKSTEPS = SLICESTEPS = 1
+    chunkBytes = stepBytes;
+    sliceBytes = stepBytes;
+    g->slicesPerChunk = 1;
+    g->fifoSlots = 8;
+  } else {  // CHUNKSTEPS 4, SLICESTEPS 2
+    chunkBytes = stepBytes * 4;
+    sliceBytes = stepBytes * 2;
+    g->slicesPerChunk = 2;
+    g->fifoSlots = 4;
+  }
+  int maxCh = (int)envInt("NCCL_MAX_NCHANNELS", 32);
+  if (maxCh < 1) maxCh = 1;
+  if (maxCh > kMaxChannels) maxCh = kMaxChannels;
+  const int64_t perChannel = envInt("DFCCL_BYTES_PER_CHANNEL", (int64_t)kWgThreads * 64);
+  g->nChannels = planChannels(nBytes, maxCh, perChannel < 1 ? 1 : perChannel);
+  g->chunkElems = chunkBytes / g->elemSize;
+  g->alignElems = kAlignBytes / g->elemSize;
+  g->sliceElems = sliceBytes / g->elemSize;
+  // a slot only has to hold the largest slice this collective will ever move
+  const int64_t real0 = realChunkElems(g->kind, g->nRanks, g->nChannels, g->chunkElems, g->alignElems,
+                                       g->count > 0 ? g->count : 1, 0);
+  const int64_t maxSlice = sliceElemsFor(real0, g->slicesPerChunk, g->sliceElems);
+  g->slotBytes = roundUp64(maxSlice * g->elemSize, kAlignBytes);
+  g->chanStride = g->slotBytes * g->fifoSlots;
+}
+
+static ncclResult_t allocGroupLocked(CommGroup* g) {
+  if (g->fifo != nullptr) return ncclSuccess;
+  const size_t links = (size_t)g->nRanks * g->nChannels;
+  HIPCHECK(hipMalloc((void**)&g->fifo, links * (size_t)g->chanStride));
+  HIPCHECK(hipMalloc((void**)&g->flags, links * sizeof(ConnFlags)));
+  HIPCHECK(hipMemset(g->flags, 0, links * sizeof(ConnFlags)));
+  return ncclSuccess;
+}
+
+static ncclResult_t prepareColl(int kind, size_t count, int dtype, int op, int root, ncclComm_t comm, int collId,
+                                ofcclRankCtx_t ctx) {
+  if (ctx == nullptr || comm == nullptr) return ncclInvalidArgument;
+  if (ctx->finalized) return ncclInvalidUsage;
+  if (collId < 0 || collId >= kMaxColls || (int)ctx->colls.size() >= kMaxColls) return ncclInvalidUsage;
+  if (ctx->collIndex[collId] >= 0) return ncclInvalidUsage;
+  CommGroup* g = comm->group;
+  if (root < 0 || root >= g->nRanks) return ncclInvalidArgument;
+  if (dtype < 0 || dtype >= ncclNumTypes) return ncclInvalidArgument;
+  if (op < 0 || op >= ncclNumOps) return ncclInvalidArgument;
+  const bool reduces = (kind == kAllReduce || kind == kReduceScatter || kind == kReduce);
+  if (reduces && (op == ncclAvg || !reduceDtypeSupported(dtype))) return ncclInvalidArgument;
+  if (comm->registered) return ncclInvalidUsage;  // one communicator per collective
+  if (comm->rank != ctx->rank) return ncclInvalidArgument;
+  {
+    std::lock_guard<std::mutex> lk(g->mu);
+    if (g->device != ctx->device) return ncclInvalidUsage;
+    if (!g->planned) {
+      g->kind = kind;
+      g->dtypeUser = dtype;
+      g->op = reduces ? op : (int)ncclSum;
+      g->root = root;
+      g->countUser = count;
+      planGroup(g);
+      g->planned = true;
+    } else if (g->kind != kind || g->dtypeUser != dtype || g->countUser != count || g->root != root ||
+               (reduces && g->op != op)) {
+      return ncclInvalidArgument;  // the ranks of a communicator must describe the same collective
+    }
+  }
+  comm->registered = true;
+  ctx->collIndex[collId] = (int16_t)ctx->colls.size();
+  ctx->colls.push_back(CollReg{collId, comm});
+  return ncclSuccess;
+}
+
+// ----------------------------------------------------------------------- poller
+
+// Consumes the completion ring in ticket order and fires the callbacks
+// (startPoller / cqRead, src/enqueue_ofccl.cc:908-965,697-739).
+static void pollerLoop(ofcclRankCtx* c) {
+  uint64_t emptySpins = 0;
+  while (!c->stopPoller.load(std::memory_order_acquire)) {
+    const uint64_t v = __atomic_load_n(&c->dev.cq[c->cqRead & (kCqRing - 1)], __ATOMIC_ACQUIRE);
+    if (v != ~0ull && cqeCnt(v) == (unsigned)((c->cqRead + 1) & 0xffffffu)) {
+      const int collId = (int)cqeCollId(v);
+      c->cqRead++;
+      emptySpins = 0;
+      if (collId >= 0 && collId < kMaxColls) {
+        CallbackFunc cb = c->callbacks[collId];
+        void* args = c->cbArgs[collId];
+        c->completed.fetch_add(1, std::memory_order_acq_rel);
+        c->inflight[collId].store(0, std::memory_order_release);
+        if (cb) (void)cb(collId, args);
+      }
+      continue;
+    }
+    if (c->submitted.load(std::memory_order_acquire) == c->completed.load(std::memory_order_acquire)) {
+      std::unique_lock<std::mutex> lk(c->pollMu);
+      c->pollCv.wait_for(lk, std::chrono::milliseconds(2), [&] {
+        return c->stopPoller.load(std::memory_order_acquire) ||
+               c->submitted.load(std::memory_order_acquire) != c->completed.load(std::memory_order_acquire);
+      });
+      emptySpins = 0;
+    } else if (++emptySpins > 20000) {
+      sched_yield();
+    } else {
+      _mm_pause();
+    }
+  }
+}
+
+// --------------------------------------------------------------------- submission
+
+// Writes one entry to the host-coherent ring (sqWrite, src/enqueue_ofccl.cc:616-656).
+// Returns -1 if the ring is full.
+static int sqWrite(ofcclRankCtx* c, uint64_t sendbuff, uint64_t recvbuff, uint32_t coll, uint32_t flags) {
+  std::lock_guard<std::mutex> lk(c->sqMu);
+  const uint64_t head = __atomic_load_n(c->dev.sqHead, __ATOMIC_ACQUIRE);
+  if (c->sqTail - head >= (uint64_t)kSqCapacity) return -1;
+  const uint64_t t = c->sqTail;
+  uint64_t* w = c->dev.sq + (t & (kSqRing - 1)) * kSqeWords;
+  const uint64_t tag = sqeTag(t);
+  __atomic_store_n(&w[0], (sendbuff & kPtrMask) | tag, __ATOMIC_RELEASE);
+  __atomic_store_n(&w[1], (recvbuff & kPtrMask) | tag, __ATOMIC_RELEASE);
+  __atomic_store_n(&w[2], (uint64_t)coll | ((uint64_t)(flags & 0xffffu) << 32) | tag, __ATOMIC_RELEASE);
+  __atomic_store_n(&w[3], tag, __ATOMIC_RELEASE);
+  c->sqTail = t + 1;
+  return 0;
+}
+
+static ncclResult_t runColl(const void* sendbuff, void* recvbuff, int collId, CallbackFunc cb, void* cbArgs,
+                            ofcclRankCtx_t c) {
+  if (c == nullptr || !c->finalized) return ncclInvalidUsage;
+  if (collId < 0 || collId >= kMaxColls || c->collIndex[collId] < 0) return ncclInvalidArgument;
+  if (((uint64_t)(uintptr_t)sendbuff & ~kPtrMask) || ((uint64_t)(uintptr_t)recvbuff & ~kPtrMask))
+    return ncclInvalidArgument;
+  // one instance per collId in flight
+  int expected = 0;
+  while (!c->inflight[collId].compare_exchange_weak(expected, 1, std::memory_order_acq_rel)) {
+    expected = 0;
+    sched_yield();
+  }
+  c->callbacks[collId] = cb;
+  c->cbArgs[collId] = cbArgs;
+  c->submitted.fetch_add(1, std::memory_order_acq_rel);
+  while (sqWrite(c, (uint64_t)(uintptr_t)sendbuff, (uint64_t)(uintptr_t)recvbuff, (uint32_t)c->collIndex[collId], 0) ==
+         -1) {
+    sched_yield();
+  }
+  Daemon* d = c->daemon;
+  {
+    // wake the observer if the kernel is not resident (cheap check first)
+    std::unique_lock<std::mutex> lk(d->mu, std::try_to_lock);
+    if (!lk.owns_lock() || !d->running) {
+      if (!lk.owns_lock()) lk.lock();
+      d->cv.notify_all();
+    }
+  }
+  c->pollCv.notify_one();
+  return ncclSuccess;
+}
+
+}  // namespace dfccl
+
+using namespace dfccl;
+
+// ================================================================ communicator API
+
+DFCCL_API ncclResult_t ncclGetUniqueId(ncclUniqueId* uniqueId) {
+  if (uniqueId == nullptr) return ncclInvalidArgument;
+  memset(uniqueId, 0, sizeof(*uniqueId));
+  const uint64_t id = gNextCommId.fetch_add(1);
+  const uint64_t magic = 0x4446434c56434f4dull;  // "DFCLVCOM"
+  const uint64_t pid = (uint64_t)getpid();
+  memcpy(uniqueId->internal, &magic, 8);
+  memcpy(uniqueId->internal + 8, &id, 8);
+  memcpy(uniqueId->internal + 16, &pid, 8);
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t ncclCommInitRank(ncclComm_t* comm, int nranks, ncclUniqueId commId, int rank) {
+  if (comm == nullptr) return ncclInvalidArgument;
+  if (nranks < 1 || rank < 0 || rank >= nranks) return ncclInvalidArgument;
+  uint64_t magic, id, pid;
+  memcpy(&magic, commId.internal, 8);
+  memcpy(&id, commId.internal + 8, 8);
+  memcpy(&pid, commId.internal + 16, 8);
+  if (magic != 0x4446434c56434f4dull || pid != (uint64_t)getpid()) return ncclInvalidArgument;
+  int device = 0;
+  HIPCHECK(hipGetDevice(&device));
+  std::lock_guard<std::mutex> lk(gCommMu);
+  CommGroup* g;
+  auto it = gGroups.find(id);
+  if (it == gGroups.end()) {
+    g = new CommGroup();
+    g->id = id;
+    g->nRanks = nranks;
+    g->device = device;
+    gGroups[id] = g;
+  } else {
+    g = it->second;
+    if (g->nRanks != nranks || g->device != device) return ncclInvalidArgument;
+  }
+  g->handles++;
+  *comm = new ncclComm{g, rank, false};
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t ncclCommDestroy(ncclComm_t comm) {
+  if (comm == nullptr) return ncclSuccess;
+  CommGroup* g = comm->group;
+  bool last;
+  {
+    std::lock_guard<std::mutex> lk(gCommMu);
+    last = (--g->handles == 0);
+    if (last) gGroups.erase(g->id);
+  }
+  delete comm;
+  if (last) {
+    // freeing device memory waits for the device, which a resident daemon would
+    // block for good: hand the memory to the daemon, it frees it between launches
+    Daemon* d = nullptr;
+    {
+      std::lock_guard<std::mutex> g2(gDaemonMu);
+      auto it = gDaemons.find(g->device);
+      if (it != gDaemons.end()) d = it->second;
+    }
+    if (d != nullptr) {
+      std::lock_guard<std::mutex> lk(d->mu);
+      if (d->running) {
+        if (g->fifo) d->garbageDev.push_back(g->fifo);
+        if (g->flags) d->garbageDev.push_back(g->flags);
+        g->fifo = nullptr;
+        g->flags = nullptr;
+      }
+    }
+    if (g->fifo) (void)hipFree(g->fifo);
+    if (g->flags) (void)hipFree(g->flags);
+    delete g;
+  }
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t ncclCommCount(const ncclComm_t comm, int* count) {
+  if (comm == nullptr || count == nullptr) return ncclInvalidArgument;
+  *count = comm->group->nRanks;
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t ncclCommUserRank(const ncclComm_t comm, int* rank) {
+  if (comm == nullptr || rank == nullptr) return ncclInvalidArgument;
+  *rank = comm->rank;
+  return ncclSuccess;
+}
+
+DFCCL_API const char* ncclGetErrorString(ncclResult_t result) {
+  switch (result) {
+    case ncclSuccess: return "no error";
+    case ncclUnhandledCudaError: return "unhandled HIP error";
+    case ncclSystemError: return "unhandled system error";
+    case ncclInternalError: return "internal error";
+    case ncclInvalidArgument: return "invalid argument";
+    case ncclInvalidUsage: return "invalid usage";
+    default: return "unknown result code";
+  }
+}
+
+// ================================================================ rank context API
+
+DFCCL_API ncclResult_t ofcclInitRankCtx(ofcclRankCtx_t* rankCtx, int rank) {
+  if (rankCtx == nullptr || rank < 0) return ncclInvalidArgument;
+  int device = 0;
+  HIPCHECK(hipGetDevice(&device));
+  ofcclRankCtx* c = new ofcclRankCtx();
+  c->rank = rank;
+  c->device = device;
+  for (int i = 0; i < kMaxColls; i++) {
+    c->collIndex[i] = -1;
+    c->callbacks[i] = nullptr;
+    c->cbArgs[i] = nullptr;
+    c->inflight[i].store(0);
+  }
+  *rankCtx = c;
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t ofcclPrepareAllReduce(size_t count, ncclDataType_t datatype, ncclRedOp_t op, ncclComm_t comm,
+                                             int collId, ofcclRankCtx_t rankCtx) {
+  return prepareColl(kAllReduce, count, (int)datatype, (int)op, 0, comm, collId, rankCtx);
+}
+DFCCL_API ncclResult_t ofcclPrepareReduceScatter(size_t recvcount, ncclDataType_t datatype, ncclRedOp_t op,
+                                                 ncclComm_t comm, int collId, ofcclRankCtx_t rankCtx) {
+  return prepareColl(kReduceScatter, recvcount, (int)datatype, (int)op, 0, comm, collId, rankCtx);
+}
+DFCCL_API ncclResult_t ofcclPrepareAllGather(size_t sendcount, ncclDataType_t datatype, ncclComm_t comm, int collId,
+                                             ofcclRankCtx_t rankCtx) {
+  return prepareColl(kAllGather, sendcount, (int)datatype, (int)ncclSum, 0, comm, collId, rankCtx);
+}
+DFCCL_API ncclResult_t ofcclPrepareReduce(size_t count, ncclDataType_t datatype, ncclRedOp_t op, int root,
+                                          ncclComm_t comm, int collId, ofcclRankCtx_t rankCtx) {
+  return prepareColl(kReduce, count, (int)datatype, (int)op, root, comm, collId, rankCtx);
+}
+DFCCL_API ncclResult_t ofcclPrepareBroadcast(size_t count, ncclDataType_t datatype, int root, ncclComm_t comm,
+                                             int collId, ofcclRankCtx_t rankCtx) {
+  return prepareColl(kBroadcast, count, (int)datatype, (int)ncclSum, root, comm, collId, rankCtx);
+}
+DFCCL_API ncclResult_t ofcclPrepareBcast(size_t count, ncclDataType_t datatype, int root, ncclComm_t comm, int collId,
+                                         ofcclRankCtx_t rankCtx) {
+  return ofcclPrepareBroadcast(count, datatype, root, comm, collId, rankCtx);
+}
+
+DFCCL_API ncclResult_t ofcclFinalizeRankCtx7StartHostThrds(ofcclRankCtx_t c) {
+  if (c == nullptr) return ncclInvalidArgument;
+  if (c->finalized) return ncclInvalidUsage;
+  HIPCHECK(hipSetDevice(c->device));
+  Daemon* d = nullptr;
+  ncclResult_t r = getDaemon(c->device, &d);
+  if (r != ncclSuccess) return r;
+  const int nColls = (int)c->colls.size();
+  const int nCollsAlloc = nColls > 0 ? nColls : 1;
+
+  // per-collective plans of this rank
+  std::vector<CollPlan> plans((size_t)nCollsAlloc);
+  memset(plans.data(), 0, plans.size() * sizeof(CollPlan));
+  HIPCHECK(hipMalloc((void**)&c->doneCounters, (size_t)nCollsAlloc * sizeof(uint64_t)));
+  HIPCHECK(hipMemset(c->doneCounters, 0, (size_t)nCollsAlloc * sizeof(uint64_t)));
+  int maxCh = 1;
+  for (int i = 0; i < nColls; i++) {
+    CommGroup* g = c->colls[i].comm->group;
+    {
+      std::lock_guard<std::mutex> lk(g->mu);
+      r = allocGroupLocked(g);
+      if (r != ncclSuccess) return r;
+    }
+    CollPlan& p = plans[i];
+    const int n = g->nRanks, rank = c->rank, prev = (rank + n - 1) % n;
+    p.kind = g->kind; p.dtype = g->dtype; p.op = g->op; p.root = g->root;
+    p.nRanks = n; p.rank = rank; p.nChannels = g->nChannels; p.collId = c->colls[i].collId;
+    p.count = g->count; p.chunkElems = g->chunkElems; p.alignElems = g->alignElems; p.sliceElems = g->sliceElems;
+    p.slicesPerChunk = g->slicesPerChunk; p.fifoSlots = g->fifoSlots; p.elemSize = g->elemSize;
+    p.slotBytes = g->slotBytes; p.fifoChanStride = g->chanStride;
+    p.sendFifo = g->fifo + (size_t)rank * g->nChannels * g->chanStride;
+    p.recvFifo = g->fifo + (size_t)prev * g->nChannels * g->chanStride;
+    p.sendFlags = g->flags + (size_t)rank * g->nChannels;
+    p.recvFlags = g->flags + (size_t)prev * g->nChannels;
+    p.doneCounter = c->doneCounters + i;
+    if (g->nChannels > maxCh) maxCh = g->nChannels;
+  }
+  c->nChannels = maxCh;
+
+  // queues and per-workgroup state (sqCreate / cqCreate, src/enqueue_ofccl.cc:596-695)
+  RankDev& R = c->dev;
+  memset(&R, 0, sizeof(R));
+  R.nChannels = maxCh;
+  R.nColls = nColls;
+  R.rank = c->rank;
+  const unsigned hostFlags = hipHostMallocCoherent | hipHostMallocMapped;
+  HIPCHECK(hipHostMalloc((void**)&R.sq, (size_t)kSqRing * kSqeWords * 8, hostFlags));
+  memset(R.sq, 0, (size_t)kSqRing * kSqeWords * 8);
+  HIPCHECK(hipHostMalloc((void**)&R.sqHead, 64, hostFlags));
+  *R.sqHead = 0;
+  HIPCHECK(hipHostMalloc((void**)&R.cq, (size_t)kCqRing * 8, hostFlags));
+  memset(R.cq, 0xff, (size_t)kCqRing * 8);
+  HIPCHECK(hipHostMalloc((void**)&R.wgExit, (size_t)kMaxChannels * 4, hostFlags));
+  memset(R.wgExit, 0, (size_t)kMaxChannels * 4);
+  HIPCHECK(hipHostMalloc((void**)&R.stats, (size_t)kMaxChannels * sizeof(WgStats), hostFlags));
+  memset(R.stats, 0, (size_t)kMaxChannels * sizeof(WgStats));
+  R.ctrl = d->ctrl;
+  HIPCHECK(hipMalloc((void**)&R.mirror, (size_t)kSqRing * sizeof(DevSqe)));
+  HIPCHECK(hipMemset(R.mirror, 0, (size_t)kSqRing * sizeof(DevSqe)));
+  HIPCHECK(hipMalloc((void**)&R.mirrorTail, 64));
+  HIPCHECK(hipMemset(R.mirrorTail, 0, 64));
+  HIPCHECK(hipMalloc((void**)&R.wgFrontier, (size_t)kMaxChannels * 8));
+  HIPCHECK(hipMemset(R.wgFrontier, 0, (size_t)kMaxChannels * 8));
+  HIPCHECK(hipMalloc((void**)&R.cqTicket, 64));
+  HIPCHECK(hipMemset(R.cqTicket, 0, 64));
+  HIPCHECK(hipMalloc((void**)&R.plans, (size_t)nCollsAlloc * sizeof(CollPlan)));
+  HIPCHECK(hipMemcpy(R.plans, plans.data(), (size_t)nCollsAlloc * sizeof(CollPlan), hipMemcpyHostToDevice));
+  HIPCHECK(hipMalloc((void**)&R.dyn, (size_t)maxCh * nCollsAlloc * sizeof(DynCtx)));
+  HIPCHECK(hipMemset(R.dyn, 0, (size_t)maxCh * nCollsAlloc * sizeof(DynCtx)));
+  HIPCHECK(hipMalloc((void**)&R.saved, (size_t)maxCh * sizeof(WgSaved)));
+  HIPCHECK(hipMemset(R.saved, 0, (size_t)maxCh * sizeof(WgSaved)));
+
+  // attach to the device daemon; a resident kernel has to leave first so that
+  // the next launch covers this rank's workgroups
+  {
+    std::unique_lock<std::mutex> lk(d->mu);
+    int slot = -1;
+    for (int s = 0; s < kMaxRankSlots; s++)
+      if (d->slots[s] == nullptr) { slot = s; break; }
+    if (slot < 0) return ncclInvalidUsage;
+    d->readKnobs();
+    d->quiesceLocked(lk);
+    d->slots[slot] = c;
+    d->nActive++;
+    c->slot = slot;
+    c->daemon = d;
+    c->finalized = true;
+    d->cv.notify_all();
+  }
+  c->poller = std::thread([c] { pollerLoop(c); });
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t ofcclPrepareDone(ofcclRankCtx_t c) {
+  ncclResult_t r = ofcclFinalizeRankCtx7StartHostThrds(c);
+  if (r != ncclSuccess) return r;
+  Daemon* d = c->daemon;
+  std::lock_guard<std::mutex> lk(d->mu);
+  if (!d->running) {
+    d->launchRequested = true;
+    d->cv.notify_all();
+  }
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t ofcclDestroy(ofcclRankCtx_t c) {
+  if (c == nullptr) return ncclInvalidArgument;
+  if (c->finalized) {
+    Daemon* d = c->daemon;
+    bool quitSent = false;
+    bool lastRank = false;
+    const auto deadline = std::chrono::steady_clock::now() + std::chrono::seconds(20);
+    for (;;) {
+      std::unique_lock<std::mutex> lk(d->mu);
+      bool out = !d->running;
+      if (!out) {
+        // out of the kernel once every workgroup of the rank has written its exit word in this launch
+        out = true;
+        for (int ch = 0; ch < c->nChannels; ch++) {
+          const uint32_t w = __atomic_load_n(&c->dev.wgExit[ch], __ATOMIC_ACQUIRE);
+          if ((w >> 4) != d->epoch || (w & 0xf) == kExitNone) { out = false; break; }
+        }
+      }
+      if (out) {
+        d->slots[c->slot] = nullptr;
+        d->nActive--;
+        lastRank = (d->nActive == 0);
+        break;
+      }
+      if (!quitSent) {
+        lk.unlock();
+        // the quit entry (src/enqueue_ofccl.cc:1593-1594)
+        c->submitted.fetch_add(1, std::memory_order_acq_rel);
+        while (sqWrite(c, 0, 0, 0, kSqeFlagQuit) == -1) sched_yield();
+        quitSent = true;
+        continue;
+      }
+      if (std::chrono::steady_clock::now() > deadline) {
+        fprintf(stderr, "dfccl: rank %d did not leave the daemon, aborting the daemon\n", c->rank);
+        __atomic_store_n(d->ctrl, kCtrlAbort, __ATOMIC_RELEASE);
+        d->cv.wait_for(lk, std::chrono::seconds(10), [&] { return !d->running; });
+        d->slots[c->slot] = nullptr;
+        d->nActive--;
+        lastRank = (d->nActive == 0);
+        break;
+      }
+      lk.unlock();
+      usleep(50);
+    }
+    c->stopPoller.store(true, std::memory_order_release);
+    c->pollCv.notify_all();
+    if (c->poller.joinable()) c->poller.join();
+
+    RankDev& R = c->dev;
+    void* devPtrs[] = {R.mirror, R.mirrorTail, R.wgFrontier, R.cqTicket, R.plans, R.dyn, R.saved, c->doneCounters};
+    void* hostPtrs[] = {R.sq, R.sqHead, R.cq, R.wgExit, R.stats};
+    if (lastRank) {
+      destroyDaemon(d);
+      for (void* p : devPtrs) if (p) (void)hipFree(p);
+      for (void* p : hostPtrs) if (p) (void)hipHostFree(p);
+    } else {
+      std::lock_guard<std::mutex> lk(d->mu);
+      if (d->running) {
+        for (void* p : devPtrs) if (p) d->garbageDev.push_back(p);
+        for (void* p : hostPtrs) if (p) d->garbageHost.push_back(p);
+      } else {
+        for (void* p : devPtrs) if (p) (void)hipFree(p);
+        for (void* p : hostPtrs) if (p) (void)hipHostFree(p);
+      }
+    }
+  }
+  for (auto& reg : c->colls) reg.comm->registered = false;
+  delete c;
+  return ncclSuccess;
+}
+
+// ======================================================================== run API
+
+DFCCL_API ncclResult_t ofcclRunAllReduce(const void* sendbuff, void* recvbuff, int collId, CallbackFunc callback,
+                                         void* callbackArgs, ofcclRankCtx_t rankCtx) {
+  return runColl(sendbuff, recvbuff, collId, callback, callbackArgs, rankCtx);
+}
+DFCCL_API ncclResult_t ofcclRunReduceScatter(const void* sendbuff, void* recvbuff, int collId, CallbackFunc callback,
+                                             void* callbackArgs, ofcclRankCtx_t rankCtx) {
+  return runColl(sendbuff, recvbuff, collId, callback, callbackArgs, rankCtx);
+}
+DFCCL_API ncclResult_t ofcclRunAllGather(const void* sendbuff, void* recvbuff, int collId, CallbackFunc callback,
+                                         void* callbackArgs, ofcclRankCtx_t rankCtx) {
+  return runColl(sendbuff, recvbuff, collId, callback, callbackArgs, rankCtx);
+}
+DFCCL_API ncclResult_t ofcclRunReduce(const void* sendbuff, void* recvbuff, int collId, CallbackFunc callback,
+                                      void* callbackArgs, ofcclRankCtx_t rankCtx) {
+  return runColl(sendbuff, recvbuff, collId, callback, callbackArgs, rankCtx);
+}
+DFCCL_API ncclResult_t ofcclRunBroadcast(const void* sendbuff, void* recvbuff, int collId, CallbackFunc callback,
+                                         void* callbackArgs, ofcclRankCtx_t rankCtx) {
+  return runColl(sendbuff, recvbuff, collId, callback, callbackArgs, rankCtx);
+}
+DFCCL_API ncclResult_t ofcclRunBcast(void* buff, int collId, CallbackFunc callback, void* callbackArgs,
+                                     ofcclRankCtx_t rankCtx) {
+  return runColl(buff, buff, collId, callback, callbackArgs, rankCtx);  // in place (ofccl_broadcast.cc:37-44)
+}
+
+// ================================================================== introspection
+
+DFCCL_API ncclResult_t dfcclGetStats(ofcclRankCtx_t c, dfcclStats* out) {
+  if (c == nullptr || out == nullptr) return ncclInvalidArgument;
+  memset(out, 0, sizeof(*out));
+  if (!c->finalized) return ncclInvalidUsage;
+  for (int ch = 0; ch < c->nChannels; ch++) {
+    const WgStats* s = &c->dev.stats[ch];
+    out->sqesRead += __atomic_load_n(&s->sqesRead, __ATOMIC_ACQUIRE);
+    out->cqesWritten += __atomic_load_n(&s->cqesWritten, __ATOMIC_ACQUIRE);
+    out->ctxSaves += __atomic_load_n(&s->ctxSaves, __ATOMIC_ACQUIRE);
+    out->ctxLoads += __atomic_load_n(&s->ctxLoads, __ATOMIC_ACQUIRE);
+    out->voluntaryQuits += __atomic_load_n(&s->voluntaryQuits, __ATOMIC_ACQUIRE);
+    out->forcedQuits += __atomic_load_n(&s->forcedQuits, __ATOMIC_ACQUIRE);
+    out->slicesMoved += __atomic_load_n(&s->slicesMoved, __ATOMIC_ACQUIRE);
+  }
+  std::lock_guard<std::mutex> lk(c->daemon->mu);
+  out->daemonLaunches = c->daemon->launches;
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t dfcclGetCollGeometry(ofcclRankCtx_t c, int collId, dfcclCollGeometry* geom) {
+  if (c == nullptr || geom == nullptr) return ncclInvalidArgument;
+  if (collId < 0 || collId >= kMaxColls || c->collIndex[collId] < 0) return ncclInvalidArgument;
+  const CommGroup* g = c->colls[(size_t)c->collIndex[collId]].comm->group;
+  geom->nRanks = g->nRanks;
+  geom->nChannels = g->nChannels;
+  geom->chunkElems = g->chunkElems;
+  geom->alignElems = g->alignElems;
+  geom->sliceElems = g->sliceElems;
+  geom->slicesPerChunk = g->slicesPerChunk;
+  geom->fifoSlots = g->fifoSlots;
+  return ncclSuccess;
+}

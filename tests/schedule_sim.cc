@@ -1,0 +1,114 @@
+// Host-side interpreter of the ring schedule the daemon kernel executes
+// (dfccl_amd/csrc/ring_schedule.h): every virtual rank is a resumable state
+// machine (loop, step, slice) that blocks on the same head / tail counters and
+// uses the same FIFO slot indexing as the device code.  Element arithmetic is
+// the oracle's.  Test infrastructure: lets the CPU suite check the schedule,
+// the slice sizing and the flow control against the oracle without a GPU.
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "../dfccl_amd/csrc/ring_schedule.h"
+#include "../oracle/dfccl_oracle.h"
+
+using namespace dfccl;
+
+namespace {
+struct Link {            // FIFO from rank r to rank (r+1)%n, one per channel
+  std::vector<char> data;
+  uint64_t tail = 0, head = 0;
+};
+struct RankState {
+  int64_t grid = 0;
+  int step = 0, slice = 0;
+  uint64_t sendStep = 0, recvStep = 0;
+  bool done = false;
+};
+}  // namespace
+
+extern "C" int sim_collective(int kind, int dtype, int op, int n, int nChannels, int64_t chunkElems,
+                              int64_t alignElems, int64_t sliceElems, int slicesPerChunk, int fifoSlots,
+                              int64_t count, int root, const void* const* send, void* const* recv,
+                              int64_t* maxSliceSeen) {
+  const int es = (kind == kAllGather || kind == kBroadcast) ? 1 : orc_type_size(dtype);
+  if (kind == kAllGather || kind == kBroadcast) { count *= orc_type_size(dtype); dtype = ORC_I8; }
+  const int64_t real0 = realChunkElems(kind, n, nChannels, chunkElems, alignElems, count > 0 ? count : 1, 0);
+  const int64_t slotElems = sliceElemsFor(real0, slicesPerChunk, sliceElems);
+  *maxSliceSeen = 0;
+  for (int ch = 0; ch < nChannels; ch++) {
+    std::vector<Link> links(n);
+    for (auto& l : links) l.data.resize((size_t)slotElems * es * fifoSlots);
+    std::vector<RankState> st(n);
+    const int64_t loop = loopElems(kind, n, nChannels, chunkElems);
+    const int nsteps = stepsPerLoop(kind, n);
+    int remaining = n;
+    for (auto& s : st) if (count <= 0) { s.done = true; remaining--; }
+    long guard = 0;
+    while (remaining > 0) {
+      bool any = false;
+      for (int r = 0; r < n; r++) {
+        RankState& s = st[r];
+        if (s.done) continue;
+        // run rank r until it blocks (this is one "visit" of the scheduler)
+        for (;;) {
+          if (s.grid >= count) { s.done = true; remaining--; break; }
+          const int64_t real = realChunkElems(kind, n, nChannels, chunkElems, alignElems, count, s.grid);
+          const char* sb = (const char*)send[r];
+          char* rb = (char*)recv[r];
+          int inPlace = (kind == kAllGather) ? (sb == rb + (int64_t)r * count * es) : (sb == rb);
+          StepDesc d = describeStep(kind, n, r, root, nChannels, ch, count, s.grid, real, s.step, inPlace);
+          bool advanceStep = false;
+          if (d.nelem <= 0) advanceStep = true;
+          else {
+            const int64_t sl = sliceElemsFor(d.nelem, slicesPerChunk, sliceElems);
+            if (sl > *maxSliceSeen) *maxSliceSeen = sl;
+            if (sl > slotElems) return -2;  // a slice would not fit its FIFO slot
+            const int64_t off = (int64_t)s.slice * sl;
+            if (off >= d.nelem) advanceStep = true;
+            else {
+              const int64_t len = (d.nelem - off < sl) ? d.nelem - off : sl;
+              Link& in = links[(r + n - 1) % n];
+              Link& out = links[r];
+              if (d.recv && in.tail < s.recvStep + 1) break;                          // wait for data
+              if (d.send && out.head + (uint64_t)fifoSlots < s.sendStep + 1) break;    // wait for space
+              const char* fifoIn = d.recv ? in.data.data() + (s.recvStep % fifoSlots) * slotElems * es : nullptr;
+              char* fifoOut = d.send ? out.data.data() + (s.sendStep % fifoSlots) * slotElems * es : nullptr;
+              const char* s0; const char* s1 = nullptr; char* d0; char* d1 = nullptr;
+              if (d.useIn) { s0 = sb + (d.inOff + off) * es; s1 = fifoIn; } else s0 = fifoIn;
+              if (d.useOut) { d0 = rb + (d.outOff + off) * es; d1 = fifoOut; } else d0 = fifoOut;
+              if (s0 && d0) {
+                std::vector<char> tmp((size_t)len * es);
+                if (s1) { const void* srcs[2] = {s0, s1}; orc_reduce_copy(dtype, op, 2, srcs, tmp.data(), (size_t)len); }
+                else memcpy(tmp.data(), s0, (size_t)len * es);
+                memcpy(d0, tmp.data(), (size_t)len * es);
+                if (d1) memcpy(d1, tmp.data(), (size_t)len * es);
+              }
+              if (d.send) { s.sendStep++; out.tail = s.sendStep; }
+              if (d.recv) { s.recvStep++; in.head = s.recvStep; }
+              s.slice++;
+              any = true;
+              continue;
+            }
+          }
+          if (advanceStep) {
+            s.slice = 0;
+            if (++s.step >= nsteps) { s.step = 0; s.grid += loop; }
+            any = true;
+          }
+        }
+      }
+      if (!any && remaining > 0) return -1;  // deadlock: nobody can move
+      if (++guard > 100000000L) return -3;
+    }
+  }
+  return 0;
+}
+
+extern "C" int sim_plan_channels(int64_t nBytes, int maxChannels, int64_t bytesPerChannel) {
+  return planChannels(nBytes, maxChannels, bytesPerChannel);
+}
+extern "C" uint64_t sim_cqe_encode(unsigned blk, unsigned cnt, unsigned coll) { return cqeEncode(blk, cnt, coll); }
+extern "C" void sim_cqe_decode(uint64_t v, unsigned* blk, unsigned* cnt, unsigned* coll) {
+  *blk = cqeBlk(v); *cnt = cqeCnt(v); *coll = cqeCollId(v);
+}
