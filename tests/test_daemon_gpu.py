@@ -1,0 +1,347 @@
+"""Parity of the collectives run through the daemon kernel (ofccl C ABI) against
+the CPU oracle, plus the scheduler's invariants: preemption and resume are
+bit-exact, out-of-order submission completes, the kernel leaves when idle and is
+relaunched, contexts can be destroyed and recreated.
+
+Bit-exact everywhere: integer ops by nature, float ops because the oracle
+reproduces the ring's per-chunk rank order from the geometry the library reports."""
+import os
+import threading
+import time
+
+import numpy as np
+import pytest
+import torch
+
+import datagen
+import dfccl_oracle as orc
+from gpu_util import TORCH_OF, geom_of, to_gpu, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _bounded_daemon(monkeypatch):
+    # a daemon that would otherwise stay resident leaves (and is relaunched on demand) every 10 s
+    monkeypatch.setenv("DFCCL_DAEMON_MAX_MS", "10000")
+    yield
+
+
+def oracle_run(kind, dtype, op, g, root, sends):
+    if kind == "all_reduce":
+        return orc.all_reduce(dtype, op, g, sends)
+    if kind == "reduce_scatter":
+        return orc.reduce_scatter(dtype, op, g, sends)
+    if kind == "all_gather":
+        return orc.all_gather(dtype, g, sends)
+    if kind == "reduce":
+        return orc.reduce(dtype, op, g, root, sends)
+    return orc.broadcast(dtype, g, root, sends)
+
+
+def make_buffers(kind, dtype, n, count, seed, **kw):
+    send_len = count * n if kind == "reduce_scatter" else count
+    recv_len = count * n if kind == "all_gather" else count
+    sends_np = [datagen.make(dtype, seed + r, send_len, **kw) for r in range(n)]
+    sends = [to_gpu(dtype, s) for s in sends_np]
+    recvs = [torch.zeros(recv_len, dtype=TORCH_OF[dtype], device="cuda:0") for _ in range(n)]
+    torch.cuda.current_stream().synchronize()
+    return sends_np, sends, recvs
+
+
+def check(kind, dtype, op, n, count, root=0, seed=100, reps=1, **kw):
+    from dfccl_amd.ring import VirtualRing
+    with VirtualRing(n) as ring:
+        ring.prepare(0, kind, count, dtype, op, root)
+        ring.finalize()
+        sends_np, sends, recvs = make_buffers(kind, dtype, n, count, seed, **kw)
+        want = oracle_run(kind, dtype, op, geom_of(ring, 0), root, sends_np)
+        for _ in range(reps):
+            ring.run(0, sends, recvs, timeout=30)
+            for r in range(n):
+                if kind == "reduce" and r != root:
+                    continue
+                assert np.array_equal(to_np(dtype, recvs[r]), want[r]), f"rank {r}"
+            for t in recvs:
+                t.zero_()
+            torch.cuda.current_stream().synchronize()
+        return ring.stats()
+
+
+@pytest.mark.parametrize("n", [2, 3, 4, 8])
+@pytest.mark.parametrize("count", [1, 37, 2048, 100003, 1 << 20])
+def test_all_reduce_fp32_sum_sizes_and_ranks(n, count):
+    check("all_reduce", orc.F32, orc.SUM, n, count, reps=2)
+
+
+@pytest.mark.parametrize("dtype", orc.DTYPES)
+@pytest.mark.parametrize("op", orc.OPS)
+def test_all_reduce_every_dtype_and_op(dtype, op):
+    check("all_reduce", dtype, op, 4, 300001, small_ints=(op == orc.PROD), seed=200 + dtype)
+
+
+@pytest.mark.parametrize("kind", ["reduce_scatter", "all_gather", "reduce", "broadcast"])
+@pytest.mark.parametrize("n,count", [(2, 1000), (4, 65537), (8, 1 << 18), (3, 5)])
+def test_other_collectives_bf16(kind, n, count):
+    check(kind, orc.BF16, orc.SUM, n, count, root=n - 1, seed=300)
+
+
+@pytest.mark.parametrize("kind", ["reduce_scatter", "reduce"])
+@pytest.mark.parametrize("dtype,op", [(orc.I8, orc.MIN), (orc.I32, orc.SUM), (orc.F16, orc.MAX), (orc.F32, orc.PROD)])
+def test_reducing_collectives_dtypes(kind, dtype, op):
+    check(kind, dtype, op, 4, 70001, root=1, seed=400)
+
+
+def test_config2_geometry_ring_all_reduce_8_ranks_bf16():
+    # 8 virtual ranks, bf16 Sum, 512 KiB chunks (262,144 elements), normal(0,1); 4 Mi elements per
+    # rank here so that the host oracle finishes in seconds (the full 64 MiB shape is in the benchmark)
+    from dfccl_amd.ring import VirtualRing
+    n, count = 8, 4 << 20
+    with VirtualRing(n) as ring:
+        ring.prepare(0, "all_reduce", count, orc.BF16, orc.SUM)
+        ring.finalize()
+        g = ring.ctxs[0].geometry(0)
+        assert g.chunkElems == 262144 and g.nChannels == 32
+        sends_np, sends, recvs = make_buffers("all_reduce", orc.BF16, n, count, 2)
+        want = orc.all_reduce(orc.BF16, orc.SUM, geom_of(ring, 0), sends_np)
+        ring.run(0, sends, recvs, timeout=30)
+        for r in range(n):
+            assert np.array_equal(to_np(orc.BF16, recvs[r]), want[r])
+        # and within 1 bf16 ulp (2^-8 relative) per accumulated term of the exact sum, the ulp taken at the
+        # largest magnitude a partial sum can reach
+        exact = sum(orc.bf16_bits_to_f32(s).astype(np.float64) for s in sends_np)
+        bound = sum(np.abs(orc.bf16_bits_to_f32(s).astype(np.float64)) for s in sends_np)
+        got = orc.bf16_bits_to_f32(to_np(orc.BF16, recvs[0])).astype(np.float64)
+        assert np.all(np.abs(got - exact) <= (n - 1) * 2.0 ** -8 * bound + 1e-30)
+
+
+def test_in_place_all_reduce_and_bcast():
+    from dfccl_amd.ring import VirtualRing
+    n, count = 4, 50000
+    with VirtualRing(n) as ring:
+        ring.prepare(0, "all_reduce", count, orc.I32, orc.SUM)
+        ring.prepare(1, "broadcast", count, orc.I32, root=2)
+        ring.finalize()
+        sends_np, bufs, _ = make_buffers("all_reduce", orc.I32, n, count, 500)
+        ring.run(0, bufs, bufs, timeout=30)
+        want = sum(s.astype(np.int64) for s in sends_np).astype(np.int32)
+        for r in range(n):
+            assert np.array_equal(to_np(orc.I32, bufs[r]), want)
+        sends_np, bufs, _ = make_buffers("broadcast", orc.I32, n, count, 510)
+        ring.run(1, bufs, bufs, timeout=30)
+        for r in range(n):
+            assert np.array_equal(to_np(orc.I32, bufs[r]), sends_np[2])
+
+
+def test_forced_preemption_is_bit_exact(monkeypatch):
+    # force a context save after every slice: the resumed run must reproduce the
+    # un-preempted result bit for bit, for a float op whose result depends on order
+    plain = check("all_reduce", orc.F32, orc.SUM, 4, 3_000_001, seed=600)
+    assert plain["forcedQuits"] == 0
+    monkeypatch.setenv("DFCCL_FORCE_QUIT_EVERY", "1")
+    forced = check("all_reduce", orc.F32, orc.SUM, 4, 3_000_001, seed=600)
+    assert forced["forcedQuits"] > 0 and forced["ctxSaves"] >= forced["forcedQuits"]
+    # every save is matched by a later load: loads = first loads (one per workgroup and instance) + saves
+    assert forced["ctxLoads"] >= forced["ctxSaves"]
+    monkeypatch.setenv("DFCCL_FORCE_QUIT_EVERY", "3")
+    check("reduce_scatter", orc.BF16, orc.SUM, 8, 400_000, seed=610)
+    check("all_gather", orc.I8, orc.SUM, 3, 1_000_003, seed=620)
+    check("reduce", orc.F16, orc.SUM, 4, 900_001, root=3, seed=630)
+
+
+def test_tiny_spin_budget_preempts_and_still_completes(monkeypatch):
+    monkeypatch.setenv("BASE_CTX_SWITCH_THRESHOLD", "1")
+    monkeypatch.setenv("NUM_TRY_TASKQ_HEAD", "1")
+    monkeypatch.setenv("RECV_SUCCESS_FACTOR", "0")
+    stats = check("all_reduce", orc.I32, orc.SUM, 8, 2_000_000, seed=700, reps=2)
+    assert stats["ctxSaves"] > 0
+
+
+def test_disordered_submission_completes_and_is_correct():
+    # every rank submits the same set of collectives in its own random order: a blocking
+    # library would deadlock; here every collective must complete with the right result
+    from dfccl_amd.ring import VirtualRing
+    n, ncoll = 4, 24
+    rng = np.random.RandomState(3)
+    counts = [int(c) for c in np.exp(rng.uniform(np.log(2048), np.log(1 << 20), ncoll)).astype(np.int64) // 8 * 8]
+    with VirtualRing(n) as ring:
+        for cid in range(ncoll):
+            ring.prepare(cid, "all_reduce", counts[cid], orc.F16, orc.SUM)
+        ring.finalize()
+        data = {}
+        for cid in range(ncoll):
+            data[cid] = make_buffers("all_reduce", orc.F16, n, counts[cid], 300 + cid * 4)
+        orders = [np.random.RandomState(30 + r).permutation(ncoll) for r in range(n)]
+        for i in range(ncoll):
+            for r in range(n):
+                cid = int(orders[r][i])
+                ring.submit(r, cid, data[cid][1][r], data[cid][2][r])
+        ring.wait([(r, cid) for r in range(n) for cid in range(ncoll)], timeout=60)
+        for cid in range(ncoll):
+            want = orc.all_reduce(orc.F16, orc.SUM, geom_of(ring, cid), data[cid][0])
+            for r in range(n):
+                assert np.array_equal(to_np(orc.F16, data[cid][2][r]), want[r]), (cid, r)
+        s = ring.stats()
+        assert s["cqesWritten"] == n * ncoll
+
+
+def test_rank_by_rank_submission_needs_preemption():
+    # rank 0 submits everything, then rank 1, ...: the first ranks' collectives cannot finish
+    # until the last rank has submitted, in reverse order
+    from dfccl_amd.ring import VirtualRing
+    n, ncoll, count = 3, 6, 40000
+    with VirtualRing(n) as ring:
+        for cid in range(ncoll):
+            ring.prepare(cid, "all_reduce", count, orc.I32, orc.SUM)
+        ring.finalize()
+        data = {cid: make_buffers("all_reduce", orc.I32, n, count, 800 + cid * 3) for cid in range(ncoll)}
+        for r in range(n):
+            order = range(ncoll) if r % 2 == 0 else reversed(range(ncoll))
+            for cid in order:
+                ring.submit(r, cid, data[cid][1][r], data[cid][2][r])
+            time.sleep(0.02)
+        ring.wait([(r, cid) for r in range(n) for cid in range(ncoll)], timeout=60)
+        for cid in range(ncoll):
+            want = sum(s.astype(np.int64) for s in data[cid][0]).astype(np.int32)
+            for r in range(n):
+                assert np.array_equal(to_np(orc.I32, data[cid][2][r]), want)
+        assert ring.stats()["ctxSaves"] > 0
+
+
+def test_idle_daemon_leaves_and_is_relaunched(monkeypatch):
+    from dfccl_amd.ring import VirtualRing
+    monkeypatch.setenv("TOLERANT_UNPROGRESSED_CNT", "2000")
+    n, count = 2, 10000
+    with VirtualRing(n) as ring:
+        ring.prepare(0, "all_reduce", count, orc.I32, orc.SUM)
+        ring.finalize()
+        sends_np, sends, recvs = make_buffers("all_reduce", orc.I32, n, count, 900)
+        want = (sends_np[0].astype(np.int64) + sends_np[1]).astype(np.int32)
+        ring.run(0, sends, recvs, timeout=30)
+        time.sleep(0.5)  # long enough for every workgroup to give up polling
+        torch.cuda.synchronize()  # returns only if the daemon really left the GPU
+        s1 = ring.stats()
+        assert s1["voluntaryQuits"] >= n
+        for t in recvs:
+            t.zero_()
+        torch.cuda.current_stream().synchronize()
+        ring.run(0, sends, recvs, timeout=30)
+        assert np.array_equal(to_np(orc.I32, recvs[1]), want)
+        assert ring.stats()["daemonLaunches"] >= s1["daemonLaunches"] + 1
+
+
+def test_voluntary_quit_with_collectives_in_flight(monkeypatch):
+    # rank 1 submits late: rank 0's workgroups give up, save their task queue, and pick the
+    # collective up again after the relaunch
+    from dfccl_amd.ring import VirtualRing
+    monkeypatch.setenv("TOLERANT_UNPROGRESSED_CNT", "300")
+    n, count = 2, 200000
+    with VirtualRing(n) as ring:
+        ring.prepare(0, "all_reduce", count, orc.F32, orc.SUM)
+        ring.finalize()
+        sends_np, sends, recvs = make_buffers("all_reduce", orc.F32, n, count, 910)
+        ring.submit(0, 0, sends[0], recvs[0])
+        time.sleep(0.3)
+        ring.submit(1, 0, sends[1], recvs[1])
+        ring.wait([(0, 0), (1, 0)], timeout=30)
+        want = orc.all_reduce(orc.F32, orc.SUM, geom_of(ring, 0), sends_np)
+        for r in range(n):
+            assert np.array_equal(to_np(orc.F32, recvs[r]), want[r])
+        s = ring.stats()
+        assert s["voluntaryQuits"] > 0 and s["daemonLaunches"] > 1
+
+
+def test_contexts_can_be_destroyed_and_recreated():
+    for i in range(3):
+        check("all_reduce", orc.I32, orc.SUM, 2 + i, 10000 + i, seed=950 + i)
+
+
+def test_second_ring_joins_a_running_daemon():
+    from dfccl_amd.ring import VirtualRing
+    count = 30000
+    with VirtualRing(2) as a:
+        a.prepare(0, "all_reduce", count, orc.I32, orc.SUM)
+        a.finalize()
+        sa_np, sa, ra = make_buffers("all_reduce", orc.I32, 2, count, 960)
+        a.run(0, sa, ra, timeout=30)
+        with VirtualRing(3) as b:  # attaches while a's daemon is resident
+            b.prepare(5, "all_reduce", count, orc.I32, orc.MAX)
+            b.finalize()
+            sb_np, sb, rb = make_buffers("all_reduce", orc.I32, 3, count, 970)
+            b.run(5, sb, rb, timeout=30)
+            a.run(0, sa, ra, timeout=30)
+            assert np.array_equal(to_np(orc.I32, rb[2]), np.maximum(np.maximum(sb_np[0], sb_np[1]), sb_np[2]))
+        a.run(0, sa, ra, timeout=30)
+        assert np.array_equal(to_np(orc.I32, ra[0]), (sa_np[0].astype(np.int64) + sa_np[1]).astype(np.int32))
+
+
+def test_callback_gets_coll_id_and_args_on_poller_thread():
+    import ctypes
+    from dfccl_amd import _lib, api
+    lib = _lib.load()
+    n, count = 2, 4096
+    comms = api.VirtualComm.create_all(n)
+    ctxs = [api.RankCtx(r) for r in range(n)]
+    try:
+        for r in range(n):
+            ctxs[r].prepare_all_reduce(count, api.ncclFloat32, api.ncclSum, comms[r], 7)
+            ctxs[r].finalize()
+        seen = []
+        done = threading.Event()
+
+        @_lib.CALLBACK
+        def cb(coll_id, args):
+            seen.append((coll_id, args, threading.get_ident()))
+            if len(seen) == n:
+                done.set()
+            return 0
+
+        bufs = [torch.ones(count, device="cuda:0") for _ in range(n)]
+        torch.cuda.current_stream().synchronize()
+        for r in range(n):
+            assert lib.ofcclRunAllReduce(bufs[r].data_ptr(), bufs[r].data_ptr(), 7, cb, ctypes.c_void_p(0x1000 + r),
+                                         ctxs[r].handle) == 0
+        assert done.wait(30)
+        assert sorted(a for _, a, _ in seen) == [0x1000, 0x1001]
+        assert all(c == 7 for c, _, _ in seen)
+        assert all(t != threading.get_ident() for _, _, t in seen)
+        assert torch.equal(bufs[0], torch.full((count,), 2.0, device="cuda:0"))
+    finally:
+        for c in ctxs:
+            c.destroy()
+        for c in comms:
+            c.destroy()
+
+
+def test_prepare_validation_follows_the_reference():
+    from dfccl_amd import api
+    comms = api.VirtualComm.create_all(2)
+    other = api.VirtualComm.create_all(2)
+    ctx = api.RankCtx(0)
+    try:
+        with pytest.raises(api.NcclError) as e:
+            ctx.prepare_all_reduce(16, api.ncclFloat32, api.ncclSum, comms[0], 2000)  # collId out of range
+        assert e.value.code == 5
+        with pytest.raises(api.NcclError) as e:
+            ctx.prepare_reduce(16, api.ncclFloat32, api.ncclSum, 2, comms[0], 1)  # root out of range
+        assert e.value.code == 4
+        with pytest.raises(api.NcclError) as e:
+            ctx.prepare_all_reduce(16, 10, api.ncclSum, comms[0], 1)  # dtype out of range
+        assert e.value.code == 4
+        with pytest.raises(api.NcclError) as e:
+            ctx.prepare_all_reduce(16, api.ncclFloat32, 4, comms[0], 1)  # ncclAvg is not on this path
+        assert e.value.code == 4
+        ctx.prepare_all_reduce(16, api.ncclFloat32, api.ncclSum, comms[0], 1)
+        with pytest.raises(api.NcclError) as e:
+            ctx.prepare_all_reduce(16, api.ncclFloat32, api.ncclSum, comms[0], 2)  # communicator reuse
+        assert e.value.code == 5
+        with pytest.raises(api.NcclError) as e:
+            ctx.prepare_all_reduce(16, api.ncclFloat32, api.ncclSum, other[0], 1)  # collId reuse
+        assert e.value.code == 5
+        with pytest.raises(api.NcclError) as e:
+            ctx.prepare_all_reduce(16, api.ncclFloat32, api.ncclSum, other[1], 3)  # handle of another rank
+        assert e.value.code == 4
+    finally:
+        ctx.destroy()
+        for c in comms + other:
+            c.destroy()
