@@ -47,7 +47,7 @@ def bench_reduce_copy(steps, warmup, nbytes=256 << 20, k=2):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     kernel_ms = [a.elapsed_time(b) for a, b in evs]
-    ok = bool(torch.equal(dst, srcs[0] + srcs[1]))
+    ok = bool(torch.equal(dst, srcs[0] + srcs[1])) if k == 2 else bool(torch.equal(dst, srcs[0]))
     alg_bytes = (k + 1) * nbytes
     return {"wall_s": wall, "kernel_ms_avg": sum(kernel_ms) / len(kernel_ms), "kernel_ms_min": min(kernel_ms),
             "alg_bytes": alg_bytes, "correct": ok}
@@ -151,6 +151,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-daemon", action="store_true", help="skip the daemon legs")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch the 1-source copy kernel on the same buffers (known traffic: 2*N*sizeof), "
+                         "used to scale the HBM byte counters of a profiler run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; virtual ranks share it, so --gpus must be 1", file=sys.stderr)
@@ -162,6 +165,8 @@ def main():
     os.environ.setdefault("DFCCL_DAEMON_MAX_MS", "20000")
 
     rc = bench_reduce_copy(args.steps, args.warmup)
+    if args.copy_calibration:
+        bench_reduce_copy(args.steps, 1, k=1)
     gbps_kernel = rc["alg_bytes"] / (rc["kernel_ms_avg"] * 1e-3) / 1e9
     gbps_wall = rc["alg_bytes"] * args.steps / rc["wall_s"] / 1e9
     line = {
