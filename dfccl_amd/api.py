@@ -170,6 +170,12 @@ class RankCtx:
         check(self.lib.dfcclGetStats(self.handle, ctypes.byref(s)), "dfcclGetStats")
         return {n: getattr(s, n) for n, _ in Stats._fields_}
 
+    def timing_ns(self, coll_id):
+        """(submit, complete) steady-clock ns of coll_id's last instance, taken inside the library."""
+        a, b = ctypes.c_uint64(), ctypes.c_uint64()
+        check(self.lib.dfcclGetCollTiming(self.handle, coll_id, ctypes.byref(a), ctypes.byref(b)), "dfcclGetCollTiming")
+        return a.value, b.value
+
     def geometry(self, coll_id):
         g = CollGeometry()
         check(self.lib.dfcclGetCollGeometry(self.handle, coll_id, ctypes.byref(g)), "dfcclGetCollGeometry")

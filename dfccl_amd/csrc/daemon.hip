@@ -27,7 +27,7 @@
 
 namespace dfccl {
 
-constexpr int kDaemonUnroll = 4;
+constexpr int kDaemonUnroll = 1;  // see reduce_copy.hip: shallow unrolling keeps DRAM accesses ordered
 enum RunStatus : int { kRunDone = 0, kRunPreempted = 1 };
 
 struct WgShared {

@@ -44,6 +44,11 @@ namespace dfccl {
     }                                                                                                   \
   } while (0)
 
+static inline uint64_t nowNs() {
+  return (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(
+             std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
 static int64_t envInt(const char* name, int64_t dflt) {
   const char* v = getenv(name);
   if (v == nullptr || *v == 0) return dflt;
@@ -129,6 +134,8 @@ struct ofcclRankCtx {
   CallbackFunc callbacks[dfccl::kMaxColls];
   void* cbArgs[dfccl::kMaxColls];
   std::atomic<int> inflight[dfccl::kMaxColls];
+  uint64_t submitNs[dfccl::kMaxColls];    // steady-clock time the last instance was queued
+  uint64_t completeNs[dfccl::kMaxColls];  // steady-clock time its completion entry was seen by the poller
   std::atomic<uint64_t> submitted{0}, completed{0};
   std::thread poller;
   std::atomic<bool> stopPoller{false};
@@ -435,12 +442,14 @@ static void pollerLoop(ofcclRankCtx* c) {
   while (!c->stopPoller.load(std::memory_order_acquire)) {
     const uint64_t v = __atomic_load_n(&c->dev.cq[c->cqRead & (kCqRing - 1)], __ATOMIC_ACQUIRE);
     if (v != ~0ull && cqeCnt(v) == (unsigned)((c->cqRead + 1) & 0xffffffu)) {
+      const uint64_t tSeen = nowNs();
       const int collId = (int)cqeCollId(v);
       c->cqRead++;
       emptySpins = 0;
       if (collId >= 0 && collId < kMaxColls) {
         CallbackFunc cb = c->callbacks[collId];
         void* args = c->cbArgs[collId];
+        c->completeNs[collId] = tSeen;
         c->completed.fetch_add(1, std::memory_order_acq_rel);
         c->inflight[collId].store(0, std::memory_order_release);
         if (cb) (void)cb(collId, args);
@@ -500,6 +509,9 @@ static ncclResult_t runColl(const void* sendbuff, void* recvbuff, int collId, Ca
          -1) {
     sched_yield();
   }
+  // written before the completion can be consumed only in practice (the device round trip takes microseconds);
+  // readers take it after the callback
+  c->submitNs[collId] = nowNs();
   Daemon* d = c->daemon;
   {
     // wake the observer if the kernel is not resident (cheap check first)
@@ -632,6 +644,7 @@ DFCCL_API ncclResult_t ofcclInitRankCtx(ofcclRankCtx_t* rankCtx, int rank) {
     c->callbacks[i] = nullptr;
     c->cbArgs[i] = nullptr;
     c->inflight[i].store(0);
+    c->submitNs[i] = c->completeNs[i] = 0;
   }
   *rankCtx = c;
   return ncclSuccess;
@@ -883,6 +896,13 @@ DFCCL_API ncclResult_t dfcclGetStats(ofcclRankCtx_t c, dfcclStats* out) {
   }
   std::lock_guard<std::mutex> lk(c->daemon->mu);
   out->daemonLaunches = c->daemon->launches;
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t dfcclGetCollTiming(ofcclRankCtx_t c, int collId, uint64_t* submitNs, uint64_t* completeNs) {
+  if (c == nullptr || collId < 0 || collId >= kMaxColls || c->collIndex[collId] < 0) return ncclInvalidArgument;
+  if (submitNs) *submitNs = c->submitNs[collId];
+  if (completeNs) *completeNs = c->completeNs[collId];
   return ncclSuccess;
 }
 

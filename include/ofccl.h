@@ -171,6 +171,13 @@ typedef struct {
  * once the rank is idle. */
 ncclResult_t dfcclGetStats(ofcclRankCtx_t rankCtx, dfcclStats* stats);
 
+/* Host steady-clock times (ns) of collId's last instance on this rank: when its
+ * submission-queue entry was written and when the poller saw its completion
+ * entry, i.e. the SQE->CQE interval without the callback's own cost (the
+ * reference measures the same interval with its DEBUG_CLOCK_IO probe,
+ * src/include/collectives_ofccl.h:50-54). Read it from the callback or later. */
+ncclResult_t dfcclGetCollTiming(ofcclRankCtx_t rankCtx, int collId, uint64_t* submitNs, uint64_t* completeNs);
+
 /* Chunk geometry the library planned for collId (needed to reproduce the
  * ring's accumulation order on the host). Valid after Finalize. */
 typedef struct {
