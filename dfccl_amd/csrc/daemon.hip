@@ -5,18 +5,24 @@
 // the scheduler of the reference's daemonKernel
 // (src/collectives_ofccl/device/enqueue_ofccl_dev.cu:1026-1483) on its own:
 //
-//   poll submissions -> append to the task queue -> visit every active
-//   collective: load its context, run ring steps slice by slice until it is
-//   done or a bounded wait expires, save the context (preemption) or post the
+//   poll submissions -> append to the task queue -> find the collectives that can
+//   move -> visit them: load the context, run steps until the collective is done
+//   or a bounded wait expires, save the context (preemption) or post the
 //   completion -> repeat; leave after a long idle period, or when told to.
 //
-// Differences that come from the hardware rather than from the algorithm:
+// What is shaped by the hardware rather than by the reference:
 //  * only the rank's leader workgroup (channel 0) reads the host-coherent
-//    submission ring; one wave fetches up to 15 entries per poll (four lanes
-//    per entry, each word validated by its own tag) and mirrors them into an
-//    HBM ring the other channels read, so PCIe sees one poller per rank;
-//  * waits are done by wave 0 with a ballot over the two flag lanes (receive
-//    ready, send ready); the vote also carries the quit decision;
+//    submission ring; one wave fetches up to 15 entries per poll (four lanes per
+//    entry, each word validated by its own tag) and mirrors them into an HBM ring
+//    the other channels read, so PCIe sees one poller per rank;
+//  * every blocking point is a WaitDesc ("these counters have reached this
+//    value"); wave 0 evaluates it with one lane per counter and a ballot, and the
+//    same descriptor, saved with the context, lets the scheduler test 64 parked
+//    collectives per wave instruction instead of loading and spinning on each;
+//  * two data protocols: the reference's FIFO ring (slices staged through HBM
+//    FIFOs between neighbours) and a direct protocol in which the virtual ranks,
+//    whose buffers share one HBM, read each other's buffers in place and keep
+//    the ring's per-chunk accumulation order;
 //  * completions go to a host-coherent ring with a device-side ticket, no
 //    compare-and-swap over PCIe;
 //  * the collective's plan and resumable position live in LDS while it runs.
@@ -28,6 +34,7 @@
 namespace dfccl {
 
 constexpr int kDaemonUnroll = 1;  // see reduce_copy.hip: shallow unrolling keeps DRAM accesses ordered
+constexpr int kReadyWords = (kMaxColls + 63) / 64;
 enum RunStatus : int { kRunDone = 0, kRunPreempted = 1 };
 
 struct WgShared {
@@ -37,19 +44,25 @@ struct WgShared {
   uint64_t publishedHead;  // leader: last value written to the host's head word
   int64_t idle;            // consecutive rounds without work or progress
   int32_t numActive;
+  int32_t numReady;
   int32_t finalQuit;
   int32_t exitKind;
   int32_t ingested;
   int32_t progressedRound;
+  int32_t loadedColl;      // collective whose plan and position are in LDS, -1: none
+  int32_t statsDirty;
   // collective being run
   int32_t waitOk;
   int32_t progressed;
-  int32_t recvSuccess;
+  int32_t peersLoaded;
   int64_t threshold;
   int64_t slicesSinceLoad;
   CollPlan plan;
   DynCtx dyn;
   WgStats stats;
+  uint64_t peerSend[kMaxDirectRanks];
+  uint64_t peerRecv[kMaxDirectRanks];
+  uint64_t ready[kReadyWords];
   uint16_t taskq[kMaxColls];
 };
 
@@ -65,8 +78,25 @@ __device__ __forceinline__ uint64_t waveMin64(uint64_t v) {
   return v;
 }
 
+__device__ __forceinline__ WaitDesc noWait() {
+  WaitDesc w;
+  w.ptr = 0;
+  w.value = 0;
+  w.stride = 0;
+  w.count = 0;
+  return w;
+}
+__device__ __forceinline__ WaitDesc waitFor(const void* ptr, uint64_t value, int stride, int count) {
+  WaitDesc w;
+  w.ptr = (uint64_t)(uintptr_t)ptr;
+  w.value = value;
+  w.stride = stride;
+  w.count = count;
+  return w;
+}
+
 // Writes the workgroup's counters to host-coherent memory (thread 0).
-__device__ __forceinline__ void flushStats(const RankDev& R, const WgShared& sh, int ch) {
+__device__ __forceinline__ void flushStats(const RankDev& R, WgShared& sh, int ch) {
   WgStats* out = &R.stats[ch];
   __hip_atomic_store(&out->sqesRead, sh.stats.sqesRead, __ATOMIC_RELAXED, DFCCL_SYSTEM);
   __hip_atomic_store(&out->cqesWritten, sh.stats.cqesWritten, __ATOMIC_RELAXED, DFCCL_SYSTEM);
@@ -76,6 +106,7 @@ __device__ __forceinline__ void flushStats(const RankDev& R, const WgShared& sh,
   __hip_atomic_store(&out->forcedQuits, sh.stats.forcedQuits, __ATOMIC_RELAXED, DFCCL_SYSTEM);
   __hip_atomic_store(&out->slicesMoved, sh.stats.slicesMoved, __ATOMIC_RELAXED, DFCCL_SYSTEM);
   __hip_atomic_store(&out->spins, sh.stats.spins, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+  sh.statsDirty = 0;
 }
 
 // Leader, wave 0: fetch submissions from the host ring into the HBM mirror and
@@ -175,18 +206,47 @@ __device__ __forceinline__ void ingest(const RankDev& R, WgShared& sh, int ch, i
     if (q < avail) sh.finalQuit = 1;
     sh.ingested = consumed;
     sh.stats.sqesRead += (uint64_t)consumed;
+    sh.statsDirty = 1;
+    if (added > 0) sh.loadedColl = -1;  // a new instance may have changed the buffers of the cached context
     __hip_atomic_store(&R.wgFrontier[ch], f + (uint64_t)consumed, __ATOMIC_RELAXED, DFCCL_AGENT);
   }
 }
 
-// Wave 0: wait until the receive slot is filled and / or a send slot is free.
-// Lane 0 watches the receive link's tail, lane 1 the send link's head; the
-// ballot decides for the whole wave.  The wait is bounded: when the budget is
-// spent the collective is preempted.  (Role of waitPeer,
-// src/collectives_ofccl/device/ofccl_prims_simple.h:90-198.)
-__device__ __forceinline__ void waitPeer(const DaemonArgs& A, WgShared& sh, int ch, int lane, bool recv, bool send,
-                                         uint64_t recvStep, uint64_t sendStep) {
-  const CollPlan& P = sh.plan;
+// One lane: is this parked collective's wait condition met?
+__device__ __forceinline__ bool descMet(const WaitDesc& w) {
+  for (int i = 0; i < w.count; i++) {
+    const uint64_t* p = (const uint64_t*)(uintptr_t)(w.ptr + (uint64_t)((int64_t)i * w.stride));
+    if (__hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_AGENT) < w.value) return false;
+  }
+  return true;
+}
+
+// Wave 0: mark the collectives of the task queue that can move, 64 per pass, one
+// lane per collective, from the wait descriptors saved with their contexts.
+__device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, int ch, int lane) {
+  const int n = sh.numActive;
+  int total = 0;
+  for (int base = 0; base < n; base += 64) {
+    const int i = base + lane;
+    bool ready = false;
+    if (i < n) {
+      const DynCtx* d = &R.dyn[(size_t)ch * R.nColls + sh.taskq[i]];
+      const WaitDesc w0 = d->wait[0], w1 = d->wait[1];
+      ready = descMet(w0) && descMet(w1);
+    }
+    const uint64_t m = __ballot(ready);
+    if (lane == 0) sh.ready[base >> 6] = m;
+    total += __builtin_popcountll(m);
+  }
+  if (lane == 0) sh.numReady = total;
+}
+
+// Wave 0: wait until both conditions hold.  Lanes 0..31 watch the counters of
+// w0, lanes 32..63 those of w1; the ballot decides for the whole wave.  The wait
+// is bounded: when the budget is spent the collective is preempted.  (Role of
+// waitPeer, src/collectives_ofccl/device/ofccl_prims_simple.h:90-198.)
+__device__ __forceinline__ void waitDescs(const DaemonArgs& A, WgShared& sh, int lane, const WaitDesc& w0,
+                                          const WaitDesc& w1, bool adapt) {
   bool ok;
   int64_t spins = 0;
   const int64_t forceEvery = A.knobs.forceQuitEvery;
@@ -194,16 +254,15 @@ __device__ __forceinline__ void waitPeer(const DaemonArgs& A, WgShared& sh, int 
     ok = false;
     if (lane == 0) sh.stats.forcedQuits++;
   } else {
+    const WaitDesc& w = (lane < 32) ? w0 : w1;
+    const int idx = lane & 31;
     const uint64_t* p = nullptr;
-    if (lane == 0 && recv) p = &P.recvFlags[ch].tail;
-    if (lane == 1 && send) p = &P.sendFlags[ch].head;
+    if (idx < w.count) p = (const uint64_t*)(uintptr_t)(w.ptr + (uint64_t)((int64_t)idx * w.stride));
+    const uint64_t need = w.value;
     bool ready = (p == nullptr);
     const int64_t threshold = sh.threshold;
     for (;;) {
-      if (!ready) {
-        const uint64_t v = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_AGENT);
-        ready = (lane == 0) ? (v >= recvStep + 1) : (v + (uint64_t)P.fifoSlots >= sendStep + 1);
-      }
+      if (!ready) ready = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_AGENT) >= need;
       if (__ballot(!ready) == 0) { ok = true; break; }
       if (++spins >= threshold) { ok = false; break; }
       __builtin_amdgcn_s_sleep(1);
@@ -213,13 +272,18 @@ __device__ __forceinline__ void waitPeer(const DaemonArgs& A, WgShared& sh, int 
   if (lane == 0) {
     sh.waitOk = ok ? 1 : 0;
     sh.stats.spins += (uint64_t)spins;
-    if (ok && recv) {
-      sh.recvSuccess = 1;
+    if (ok && adapt) {
       const int64_t t = A.knobs.recvSuccessFactor * spins;
       if (t > sh.threshold) sh.threshold = t;
     }
+    if (!ok) {
+      sh.dyn.wait[0] = w0;
+      sh.dyn.wait[1] = w1;
+    }
   }
 }
+
+// ---------------------------------------------------------------- data movement
 
 template <int DT, int OP>
 __device__ __forceinline__ void moveReduce(const void* s0, const void* s1, void* d0, void* d1, size_t nbytes, int tid) {
@@ -244,18 +308,22 @@ __device__ __forceinline__ void moveReduceOp(int op, const void* s0, const void*
   }
 }
 
-// One slice: 1 or 2 sources into 1 or 2 destinations (d1 may be null).
+__device__ __forceinline__ void copySlice(const void* s0, void* d0, void* d1, size_t nbytes, int tid) {
+  const void* s[1] = {s0};
+  if (d1 != nullptr) {
+    void* d[2] = {d0, d1};
+    reduceCopyWG<kI8, kSum, 1, 2, kDaemonUnroll, false>(s, d, nbytes, tid, kWgThreads);
+  } else {
+    void* d[1] = {d0};
+    reduceCopyWG<kI8, kSum, 1, 1, kDaemonUnroll, false>(s, d, nbytes, tid, kWgThreads);
+  }
+}
+
+// One slice: 1 or 2 sources into 1 or 2 destinations (s1 / d1 may be null).
 __device__ __forceinline__ void moveSlice(int dtype, int op, const void* s0, const void* s1, void* d0, void* d1,
                                           size_t nbytes, int tid) {
   if (s1 == nullptr) {
-    const void* s[1] = {s0};
-    if (d1 != nullptr) {
-      void* d[2] = {d0, d1};
-      reduceCopyWG<kI8, kSum, 1, 2, kDaemonUnroll, false>(s, d, nbytes, tid, kWgThreads);
-    } else {
-      void* d[1] = {d0};
-      reduceCopyWG<kI8, kSum, 1, 1, kDaemonUnroll, false>(s, d, nbytes, tid, kWgThreads);
-    }
+    copySlice(s0, d0, d1, nbytes, tid);
     return;
   }
   switch (dtype) {
@@ -267,11 +335,70 @@ __device__ __forceinline__ void moveSlice(int dtype, int op, const void* s0, con
   }
 }
 
+// Direct protocol: fold n peer buffers (already offset to the chunk) in the order
+// given (n <= kMaxDirectRanks), src[0] first, into dst.  The fold keeps the ring's order for the chunk:
+// src = in[c+1], in[c+2], ..., in[c], each step rounded to the storage type.
+template <int DT, int OP>
+__device__ __forceinline__ void reduceOrdered(const char* const* src, int n, void* dst, size_t nbytes, int tid) {
+  constexpr int ES = typeSize(DT);
+  uintptr_t align = (uintptr_t)dst;
+  for (int j = 0; j < n; j++) align |= (uintptr_t)src[j];
+  size_t doneBytes = 0;
+  if ((align & 15u) == 0) {
+    const size_t npacks = nbytes >> 4;
+    for (size_t i = tid; i < npacks; i += kWgThreads) {
+      u32x4 acc;
+      {
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+          if (j < n) v[j] = loadPack<false>(src[j], i);
+        acc = v[0];
+#pragma unroll
+        for (int j = 1; j < 8; j++)
+          if (j < n) acc = packOp<DT, OP>(acc, v[j]);
+      }
+      storePack<false>(dst, i, acc);
+    }
+    doneBytes = npacks << 4;
+  }
+  const size_t first = doneBytes / ES, nelem = nbytes / ES;
+  for (size_t i = first + tid; i < nelem; i += kWgThreads) {
+    uint32_t acc = loadElem<ES>(src[0], i);
+    for (int j = 1; j < n; j++) acc = wordOp<DT, OP>(acc, loadElem<ES>(src[j], i));
+    storeElem<ES>(dst, i, acc);
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void reduceOrderedOp(int op, const char* const* src, int n, void* dst, size_t nbytes,
+                                                int tid) {
+  switch (op) {
+    case kSum: reduceOrdered<DT, kSum>(src, n, dst, nbytes, tid); break;
+    case kProd: reduceOrdered<DT, kProd>(src, n, dst, nbytes, tid); break;
+    case kMax: reduceOrdered<DT, kMax>(src, n, dst, nbytes, tid); break;
+    default: reduceOrdered<DT, kMin>(src, n, dst, nbytes, tid); break;
+  }
+}
+
+__device__ __forceinline__ void reduceOrderedAny(int dtype, int op, const char* const* src, int n, void* dst,
+                                                 size_t nbytes, int tid) {
+  switch (dtype) {
+    case kF32: reduceOrderedOp<kF32>(op, src, n, dst, nbytes, tid); break;
+    case kBF16: reduceOrderedOp<kBF16>(op, src, n, dst, nbytes, tid); break;
+    case kF16: reduceOrderedOp<kF16>(op, src, n, dst, nbytes, tid); break;
+    case kI32: reduceOrderedOp<kI32>(op, src, n, dst, nbytes, tid); break;
+    default: reduceOrderedOp<kI8>(op, src, n, dst, nbytes, tid); break;
+  }
+}
+
+// ------------------------------------------------------------- FIFO ring protocol
+
 // Runs the loaded collective from its saved position until it is done or a wait
 // expires.  Every thread takes the same path: all decisions come from LDS after
 // a barrier.  (Role of the resumable runRing bodies and genericOp; see
 // ring_schedule.h for the per-step roles.)
-__device__ __forceinline__ int runColl(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
+__device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
   const CollPlan& P = sh.plan;
   const int lane = tid & 63, wave = tid >> 6;
   const int kind = P.kind, n = P.nRanks, C = P.nChannels, es = P.elemSize;
@@ -300,7 +427,11 @@ __device__ __forceinline__ int runColl(const DaemonArgs& A, WgShared& sh, int ch
         const int64_t off = (int64_t)sl * sliceE;
         const int64_t len = (d.nelem - off < sliceE) ? d.nelem - off : sliceE;
         if (d.recv || d.send) {
-          if (wave == 0) waitPeer(A, sh, ch, lane, d.recv != 0, d.send != 0, recvStep, sendStep);
+          // receive: the slot is filled (tail >= recvStep + 1); send: a slot is free (head + slots >= sendStep + 1)
+          const WaitDesc w0 = d.recv ? waitFor(&P.recvFlags[ch].tail, recvStep + 1, 0, 1) : noWait();
+          const uint64_t needHead = (sendStep + 1 > (uint64_t)P.fifoSlots) ? sendStep + 1 - (uint64_t)P.fifoSlots : 0;
+          const WaitDesc w1 = d.send ? waitFor(&P.sendFlags[ch].head, needHead, 0, 1) : noWait();
+          if (wave == 0) waitDescs(A, sh, lane, w0, w1, d.recv != 0);
           __syncthreads();
           if (!sh.waitOk) {
             if (tid == 0) {
@@ -350,7 +481,247 @@ __device__ __forceinline__ int runColl(const DaemonArgs& A, WgShared& sh, int ch
   return kRunDone;
 }
 
-extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const DaemonArgs* __restrict__ argsPtr) {
+// ----------------------------------------------------------------- direct protocol
+
+// All-reduce in which the virtual ranks read each other's buffers in place.
+// Per loop and channel the n chunks are laid out as in the FIFO ring
+// (ring_schedule.h), chunk j is owned by rank j:
+//   step 0      reduce my own chunk from all n send buffers, in the ring's order
+//               for that chunk, into my receive buffer; then p1[me] = loops done;
+//   step s >= 1 copy chunk j = me - s from rank j's receive buffer once
+//               p1[j] says it is there; after the last one p2[me] = loops done;
+//   finally     wait until every peer's p2 covers the instance: nobody reads my
+//               buffers any more, so the completion may be posted.
+// Messages that fit the registers of one workgroup take a one-shot variant:
+// every rank folds every chunk itself (two flag exchanges in total).
+// Waits are WaitDescs, so every one of them can preempt and resume.
+__device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
+  const CollPlan& P = sh.plan;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n = P.nRanks, C = P.nChannels, es = P.elemSize, me = P.rank;
+  const int64_t count = P.count;
+  const int64_t loop = loopElems(kAllReduce, n, C, P.chunkElems);
+  const int64_t L = P.loopsPerInstance;
+  const uint64_t inst = sh.dyn.instance;
+  const uint64_t base = inst * (uint64_t)L;
+  const uint64_t sendbuff = sh.dyn.sendbuff, recvbuff = sh.dyn.recvbuff;
+  const int published = sh.dyn.slice;
+  const int peersLoaded = sh.peersLoaded;
+  const int pubStride = C * (int)sizeof(PeerPub), ctrStride = C * 8;
+  PeerPub* myPub = &P.pubs[(size_t)me * C + ch];
+  int64_t grid = sh.dyn.gridOffset;
+  int step0 = sh.dyn.step;
+  __syncthreads();  // every thread has taken its copy of the position before thread 0 changes it
+
+  if (!published && tid == 0) {
+    myPub->sendbuff = sendbuff;
+    myPub->recvbuff = recvbuff;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __hip_atomic_store(&myPub->seq, inst + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
+    sh.dyn.slice = 1;
+  }
+  if (!peersLoaded) {
+    const WaitDesc w0 = waitFor(&P.pubs[ch].seq, inst + 1, pubStride, n);
+    if (wave == 0) {
+      waitDescs(A, sh, lane, w0, noWait(), true);
+      if (sh.waitOk && lane < n) {
+        const PeerPub* pp = &P.pubs[(size_t)lane * C + ch];
+        sh.peerSend[lane] = pp->sendbuff;
+        sh.peerRecv[lane] = pp->recvbuff;
+      }
+      if (sh.waitOk && lane == 0) sh.peersLoaded = 1;
+    }
+    __syncthreads();
+    if (!sh.waitOk) return kRunPreempted;  // position unchanged
+  }
+
+  if (P.oneShot) {
+    // step 0: fold every chunk from the peers' send buffers; step 1: wait until nobody reads any more
+    const int inPlace = (sendbuff == recvbuff);
+    char* out = inPlace ? P.staging + (size_t)me * kOneShotMaxBytes : (char*)recvbuff;
+    if (step0 == 0) {
+      const int64_t real = realChunkElems(kAllReduce, n, C, P.chunkElems, P.alignElems, count, 0);
+      for (int j = 0; j < n; j++) {
+        const int64_t off = (int64_t)j * real;
+        const int64_t nelem = (count - off < real) ? count - off : real;
+        if (nelem <= 0) break;
+        const char* src[kMaxDirectRanks];
+        for (int t = 0; t < n; t++) src[t] = (const char*)sh.peerSend[(j + 1 + t) % n] + off * es;
+        reduceOrderedAny(P.dtype, P.op, src, n, out + off * es, (size_t)(nelem * es), tid);
+      }
+      __syncthreads();
+      if (tid == 0) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        __hip_atomic_store(&P.p2[(size_t)me * C + ch], base + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
+        sh.progressed = 1;
+        sh.slicesSinceLoad++;
+        sh.stats.slicesMoved++;
+      }
+    }
+    const WaitDesc w0 = waitFor(&P.p2[ch], base + 1, ctrStride, n);
+    if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
+    __syncthreads();
+    if (!sh.waitOk) {
+      if (tid == 0) {
+        sh.dyn.gridOffset = 0;
+        sh.dyn.step = 1;
+      }
+      return kRunPreempted;
+    }
+    if (inPlace) {
+      copySlice(out, (void*)recvbuff, nullptr, (size_t)(count * es), tid);
+      __syncthreads();
+    }
+    if (tid == 0) {
+      sh.dyn.instance = inst + 1;
+      sh.dyn.slice = 0;
+    }
+    return kRunDone;
+  }
+
+  for (; grid < count; grid += loop, step0 = 0) {
+    const int64_t real = realChunkElems(kAllReduce, n, C, P.chunkElems, P.alignElems, count, grid);
+    const uint64_t loopNo = base + (uint64_t)(grid / loop) + 1;
+    const int64_t chunk0 = grid + (int64_t)ch * n * real;
+    for (int s = step0; s < n; ++s) {
+      if (s == 0) {
+        const int64_t off = chunk0 + (int64_t)me * real;
+        const int64_t nelem = (count - off < real) ? count - off : real;
+        if (nelem > 0) {
+          const char* src[kMaxDirectRanks];
+          for (int t = 0; t < n; t++) src[t] = (const char*)sh.peerSend[(me + 1 + t) % n] + off * es;
+          reduceOrderedAny(P.dtype, P.op, src, n, (char*)recvbuff + off * es, (size_t)(nelem * es), tid);
+        }
+        __syncthreads();
+        if (tid == 0) {
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+          __hip_atomic_store(&P.p1[(size_t)me * C + ch], loopNo, __ATOMIC_RELAXED, DFCCL_AGENT);
+          sh.progressed = 1;
+          sh.slicesSinceLoad++;
+          sh.stats.slicesMoved++;
+        }
+      } else {
+        const int j = (me + n - s) % n;
+        const int64_t off = chunk0 + (int64_t)j * real;
+        const int64_t nelem = (count - off < real) ? count - off : real;
+        if (nelem > 0) {
+          const WaitDesc w0 = waitFor(&P.p1[(size_t)j * C + ch], loopNo, 0, 1);
+          if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
+          __syncthreads();
+          if (!sh.waitOk) {
+            if (tid == 0) {
+              sh.dyn.gridOffset = grid;
+              sh.dyn.step = s;
+            }
+            return kRunPreempted;
+          }
+          copySlice((const char*)sh.peerRecv[j] + off * es, (char*)recvbuff + off * es, nullptr, (size_t)(nelem * es),
+                    tid);
+          if (tid == 0) {
+            sh.progressed = 1;
+            sh.slicesSinceLoad++;
+            sh.stats.slicesMoved++;
+          }
+        }
+      }
+      if (s == n - 1) {
+        __syncthreads();
+        if (tid == 0) {
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+          __hip_atomic_store(&P.p2[(size_t)me * C + ch], loopNo, __ATOMIC_RELAXED, DFCCL_AGENT);
+        }
+      }
+    }
+  }
+  // nobody may still be reading my send buffer or my chunk of the receive buffer
+  {
+    const WaitDesc w0 = waitFor(&P.p2[ch], base + (uint64_t)L, ctrStride, n);
+    if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
+    __syncthreads();
+    if (!sh.waitOk) {
+      if (tid == 0) {
+        sh.dyn.gridOffset = grid;  // >= count: only this wait is left
+        sh.dyn.step = 0;
+      }
+      return kRunPreempted;
+    }
+  }
+  if (tid == 0) {
+    sh.dyn.instance = inst + 1;
+    sh.dyn.slice = 0;
+  }
+  return kRunDone;
+}
+
+__device__ __forceinline__ int runColl(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
+  if (sh.plan.proto == kProtoDirect) return runDirectAllReduce(A, sh, ch, tid);
+  return runFifo(A, sh, ch, tid);
+}
+
+// Visit one collective of the task queue: make its context resident, run it,
+// then post the completion or save the context.
+__device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int tid, int qi) {
+  const Knobs& K = A.knobs;
+  const uint32_t coll = sh.taskq[qi];
+  DynCtx* dynG = &R.dyn[(size_t)ch * R.nColls + coll];
+  if (tid == 0) {
+    if (sh.loadedColl != (int32_t)coll) {
+      sh.plan = R.plans[coll];
+      sh.dyn = *dynG;
+      sh.loadedColl = (int32_t)coll;
+      sh.peersLoaded = 0;
+      sh.stats.ctxLoads++;
+    }
+    sh.dyn.tryCnt++;
+    // spin budget of this visit: BASE * min(tries, NUM_TRY); the queue head is given NUM_TRY times more
+    const int64_t tries = sh.dyn.tryCnt < K.numTryTaskqHead ? sh.dyn.tryCnt : K.numTryTaskqHead;
+    int64_t thr = K.baseCtxSwitchThreshold * tries;
+    if (qi == 0) thr *= K.numTryTaskqHead;
+    sh.threshold = thr < 1 ? 1 : thr;
+    sh.waitOk = 1;
+    sh.progressed = 0;
+    sh.slicesSinceLoad = 0;
+    sh.dyn.wait[0] = noWait();
+    sh.dyn.wait[1] = noWait();
+    sh.statsDirty = 1;
+  }
+  __syncthreads();
+  const int status = runColl(A, sh, ch, tid);
+  __syncthreads();
+  if (tid == 0) {
+    if (sh.progressed) sh.progressedRound = 1;
+    if (status == kRunDone) {
+      // reset the position for the next instance; link counters and the instance number persist
+      sh.dyn.gridOffset = 0;
+      sh.dyn.step = 0;
+      sh.dyn.tryCnt = 0;
+      sh.dyn.active = 0;
+      if (sh.plan.proto == kProtoFifo) sh.dyn.slice = 0;
+      sh.dyn.wait[0] = noWait();
+      sh.dyn.wait[1] = noWait();
+      *dynG = sh.dyn;
+      sh.taskq[qi] = (uint16_t)kInvalidTask;
+      // completion (manipulateCQ7ResetDoneColl, enqueue_ofccl_dev.cu:773-920): the last
+      // channel to finish posts the entry; results are released to the system first
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+      const uint64_t old = __hip_atomic_fetch_add(sh.plan.doneCounter, 1ull, __ATOMIC_ACQ_REL, DFCCL_AGENT);
+      if ((old + 1) % (uint64_t)sh.plan.nChannels == 0) {
+        const uint64_t t = __hip_atomic_fetch_add(R.cqTicket, 1ull, __ATOMIC_RELAXED, DFCCL_AGENT);
+        __hip_atomic_store(&R.cq[t & (kCqRing - 1)],
+                           cqeEncode((unsigned)ch, (unsigned)(t + 1), (unsigned)sh.plan.collId), __ATOMIC_RELEASE,
+                           DFCCL_SYSTEM);
+        sh.stats.cqesWritten++;
+      }
+    } else {
+      // preempted: save the context (saveExcutingCollCtx, enqueue_ofccl_dev.cu:664-677)
+      *dynG = sh.dyn;
+      sh.stats.ctxSaves++;
+    }
+  }
+  __syncthreads();
+}
+
+extern "C" __global__ __launch_bounds__(kWgThreads, 4) void dfcclDaemonKernel(const DaemonArgs* __restrict__ argsPtr) {
   __shared__ WgShared sh;
   const DaemonArgs& A = *argsPtr;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -369,11 +740,14 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     sh.hostFrontier = S.hostFrontier;
     sh.publishedHead = ~0ull;
     sh.numActive = S.numActive;
+    sh.numReady = 0;
     sh.finalQuit = 0;
     sh.exitKind = kExitNone;
     sh.idle = 0;
     sh.ingested = 0;
     sh.progressedRound = 0;
+    sh.loadedColl = -1;
+    sh.peersLoaded = 0;
     const WgStats* hs = &R.stats[ch];
     sh.stats.sqesRead = hs->sqesRead;
     sh.stats.cqesWritten = hs->cqesWritten;
@@ -383,6 +757,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     sh.stats.forcedQuits = hs->forcedQuits;
     sh.stats.slicesMoved = hs->slicesMoved;
     sh.stats.spins = hs->spins;
+    sh.statsDirty = 0;
   }
   __syncthreads();
   for (int i = tid; i < sh.numActive; i += kWgThreads) sh.taskq[i] = S.taskq[i];
@@ -393,6 +768,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     if (wave == 0) {
       if (ch == 0) pollHost(A, R, sh, lane);
       ingest(R, sh, ch, lane);
+      scanReady(R, sh, ch, lane);
       if (lane == 0) {
         const uint32_t abortFlag = __hip_atomic_load(&A.devFlags[1], __ATOMIC_RELAXED, DFCCL_AGENT);
         const uint32_t quitFlag = __hip_atomic_load(&A.devFlags[0], __ATOMIC_RELAXED, DFCCL_AGENT);
@@ -404,9 +780,11 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
         else if (quitFlag || expired) sh.exitKind = kExitVoluntary;
         else if (sh.idle >= K.tolerantUnprogressedCnt) sh.exitKind = kExitVoluntary;
         sh.progressedRound = 0;
+        // counters go to the host when the workgroup has nothing better to do
+        if (sh.numReady == 0 && sh.statsDirty) flushStats(R, sh, ch);
       }
-      if (sh.numActive == 0 && sh.ingested == 0) {
-        // nothing to do: the leader's next poll is a PCIe round trip anyway, the others back off a little
+      if (sh.numReady == 0 && sh.ingested == 0) {
+        // nothing can move: the leader's next poll is a PCIe round trip anyway, the others back off a little
         if (ch == 0) __builtin_amdgcn_s_sleep(2);
         else __builtin_amdgcn_s_sleep(20);
       }
@@ -414,79 +792,29 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     __syncthreads();
     if (sh.exitKind != kExitNone) break;
 
-    // ---- run phase: visit every active collective once (traverseTaskQ, enqueue_ofccl_dev.cu:922-1016)
+    // ---- run phase: visit the collectives that can move, in arrival order
+    // (traverseTaskQ, enqueue_ofccl_dev.cu:922-1016)
     const int nq = sh.numActive;
-    for (int qi = 0; qi < nq; qi++) {
-      const uint32_t coll = sh.taskq[qi];
-      DynCtx* dynG = &R.dyn[(size_t)ch * R.nColls + coll];
-      if (tid == 0) {
-        sh.plan = R.plans[coll];
-        sh.dyn = *dynG;
-        sh.dyn.tryCnt++;
-        // spin budget of this visit: BASE * min(tries, NUM_TRY), the queue head is given NUM_TRY times more
-        const int64_t tries = sh.dyn.tryCnt < K.numTryTaskqHead ? sh.dyn.tryCnt : K.numTryTaskqHead;
-        int64_t thr = K.baseCtxSwitchThreshold * tries;
-        if (qi == 0) thr *= K.numTryTaskqHead;
-        sh.threshold = thr < 1 ? 1 : thr;
-        sh.waitOk = 1;
-        sh.progressed = 0;
-        sh.recvSuccess = 0;
-        sh.slicesSinceLoad = 0;
-        sh.stats.ctxLoads++;
-      }
-      __syncthreads();
-      const int status = runColl(A, sh, ch, tid);
-      __syncthreads();
-      if (tid == 0) {
-        if (sh.progressed) sh.progressedRound = 1;
-        if (status == kRunDone) {
-          // reset the position for the next instance; the link counters persist
-          dynG->gridOffset = 0;
-          dynG->step = 0;
-          dynG->slice = 0;
-          dynG->tryCnt = 0;
-          dynG->active = 0;
-          dynG->sendStep = sh.dyn.sendStep;
-          dynG->recvStep = sh.dyn.recvStep;
-          sh.taskq[qi] = (uint16_t)kInvalidTask;
-          // completion (manipulateCQ7ResetDoneColl, enqueue_ofccl_dev.cu:773-920): the
-          // last channel to finish posts the entry; results are released to the system first
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-          const uint64_t old = __hip_atomic_fetch_add(sh.plan.doneCounter, 1ull, __ATOMIC_ACQ_REL, DFCCL_AGENT);
-          if ((old + 1) % (uint64_t)sh.plan.nChannels == 0) {
-            const uint64_t t = __hip_atomic_fetch_add(R.cqTicket, 1ull, __ATOMIC_RELAXED, DFCCL_AGENT);
-            sh.stats.cqesWritten++;
-            flushStats(R, sh, ch);
-            __hip_atomic_store(&R.cq[t & (kCqRing - 1)],
-                               cqeEncode((unsigned)ch, (unsigned)(t + 1), (unsigned)sh.plan.collId), __ATOMIC_RELEASE,
-                               DFCCL_SYSTEM);
-          } else {
-            flushStats(R, sh, ch);
-          }
-        } else {
-          // preempted: save the context (saveExcutingCollCtx, enqueue_ofccl_dev.cu:664-677)
-          dynG->gridOffset = sh.dyn.gridOffset;
-          dynG->step = sh.dyn.step;
-          dynG->slice = sh.dyn.slice;
-          dynG->sendStep = sh.dyn.sendStep;
-          dynG->recvStep = sh.dyn.recvStep;
-          dynG->tryCnt = sh.dyn.tryCnt;
-          sh.stats.ctxSaves++;
+    if (sh.numReady > 0) {
+      for (int wd = 0; wd * 64 < nq; wd++) {
+        uint64_t m = sh.ready[wd];
+        while (m) {
+          const int b = (int)__builtin_ctzll(m);
+          m &= m - 1;
+          visit(A, R, sh, ch, tid, wd * 64 + b);
         }
       }
+      // drop finished collectives from the task queue, keeping arrival order
+      if (tid == 0) {
+        int w = 0;
+        for (int i = 0; i < nq; i++) {
+          const uint16_t c = sh.taskq[i];
+          if (c != (uint16_t)kInvalidTask) sh.taskq[w++] = c;
+        }
+        sh.numActive = w;
+      }
       __syncthreads();
     }
-    // ---- drop finished collectives from the task queue, keeping arrival order
-    if (tid == 0 && nq > 0) {
-      int w = 0;
-      const int total = sh.numActive;
-      for (int i = 0; i < total; i++) {
-        const uint16_t c = sh.taskq[i];
-        if (c != (uint16_t)kInvalidTask) sh.taskq[w++] = c;
-      }
-      sh.numActive = w;
-    }
-    __syncthreads();
   }
 
   // ---- leave

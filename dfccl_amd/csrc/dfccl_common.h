@@ -65,6 +65,31 @@ struct alignas(128) ConnFlags {
   uint64_t pad1[7];
 };
 
+// Direct protocol: what a rank's workgroup publishes when it starts an instance
+// of a collective, so that its peers can read its buffers in place (the role of
+// the reference's ptrExchange, src/collectives_ofccl/device/ofccl_prims_simple.h:737-869).
+struct alignas(32) PeerPub {
+  uint64_t seq;        // instances started, written last
+  uint64_t sendbuff;
+  uint64_t recvbuff;
+  uint64_t pad;
+};
+
+// A wait condition: all of `count` 64-bit counters at ptr, ptr + stride, ... have
+// reached `value`.  Every blocking point of both protocols is expressed as (at
+// most) two of these, which lets the scheduler test the readiness of a parked
+// collective without loading its context.
+struct WaitDesc {
+  uint64_t ptr;
+  uint64_t value;
+  int32_t stride;  // bytes
+  int32_t count;   // 0 = no condition
+};
+
+enum Proto : int { kProtoFifo = 0, kProtoDirect = 1 };
+constexpr int kMaxDirectRanks = 8;           // ranks whose buffers one workgroup folds in a single pass
+constexpr int kOneShotMaxBytes = 32 << 10;  // 512 threads x 4 packs of 16 bytes
+
 // Immutable plan of one collective on one rank (HBM, written at finalize).
 struct alignas(16) CollPlan {
   int32_t kind, dtype, op, root;
@@ -82,21 +107,30 @@ struct alignas(16) CollPlan {
   ConnFlags* sendFlags;    // indexed by channel
   ConnFlags* recvFlags;
   uint64_t* doneCounter;   // workgroups that finished an instance, monotonic
+  // direct protocol (peers read each other's buffers, no FIFO)
+  int32_t proto, oneShot;
+  PeerPub* pubs;           // [nRanks][nChannels]
+  uint64_t* p1;            // [nRanks][nChannels] loops whose own chunk is reduced and stored
+  uint64_t* p2;            // [nRanks][nChannels] loops whose reads of peer buffers are finished
+  char* staging;           // one-shot, in place: kOneShotMaxBytes per rank
+  int64_t loopsPerInstance;
 };
 
 // Resumable position of one collective on one workgroup (HBM). This is the
 // context a preemption saves and a resume restores.
-struct alignas(64) DynCtx {
+struct alignas(128) DynCtx {
   uint64_t sendbuff;
   uint64_t recvbuff;
   int64_t gridOffset;   // loop the workgroup is in
   int32_t step;         // ring step inside the loop
-  int32_t slice;        // slice inside the step's chunk
-  uint64_t sendStep;    // slices ever sent on the send link (persists across instances)
-  uint64_t recvStep;    // slices ever received on the receive link
+  int32_t slice;        // FIFO: slice inside the step's chunk; direct: 1 once the instance is published
+  uint64_t sendStep;    // FIFO: slices ever sent on the send link (persists across instances)
+  uint64_t recvStep;    // FIFO: slices ever received on the receive link
+  uint64_t instance;    // direct: instances completed (persists)
   int32_t tryCnt;       // scheduler visits since the instance started
   int32_t active;
-  uint64_t pad;
+  WaitDesc wait[2];     // what the collective is parked on (count 0: runnable)
+  uint64_t pad[2];
 };
 
 // Counters of one workgroup, in host-coherent memory so the host can read them

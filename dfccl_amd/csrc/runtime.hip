@@ -90,6 +90,13 @@ struct CommGroup {
   // device memory: [nRanks links][nChannels] FIFOs and flags; link r goes from rank r to rank (r+1)%n
   char* fifo = nullptr;
   ConnFlags* flags = nullptr;
+  // direct protocol
+  int proto = kProtoFifo, oneShot = 0;
+  int64_t loopsPerInstance = 0;
+  PeerPub* pubs = nullptr;   // [nRanks][nChannels]
+  uint64_t* p1 = nullptr;    // [nRanks][nChannels]
+  uint64_t* p2 = nullptr;
+  char* staging = nullptr;   // [nRanks][kOneShotMaxBytes], one-shot only
 };
 
 }  // namespace dfccl
@@ -386,14 +393,35 @@ static void planGroup(CommGroup* g) {
   const int64_t maxSlice = sliceElemsFor(real0, g->slicesPerChunk, g->sliceElems);
   g->slotBytes = roundUp64(maxSlice * g->elemSize, kAlignBytes);
   g->chanStride = g->slotBytes * g->fifoSlots;
+  // protocol: the virtual ranks of an all-reduce read each other's buffers in place unless told otherwise
+  const char* proto = getenv("DFCCL_PROTO");
+  const bool wantFifo = proto != nullptr && strcmp(proto, "fifo") == 0;
+  g->proto = (!wantFifo && g->kind == kAllReduce && g->nRanks >= 2 && g->nRanks <= kMaxDirectRanks) ? kProtoDirect
+                                                                                                   : kProtoFifo;
+  const int64_t loop = loopElems(g->kind, g->nRanks, g->nChannels, g->chunkElems);
+  g->loopsPerInstance = g->count > 0 ? divUp64(g->count, loop) : 0;
+  g->oneShot = (g->proto == kProtoDirect && g->nChannels == 1 && g->loopsPerInstance <= 1 &&
+                g->count * g->elemSize <= kOneShotMaxBytes && envInt("DFCCL_ONESHOT", 1) != 0)
+                   ? 1
+                   : 0;
 }
 
 static ncclResult_t allocGroupLocked(CommGroup* g) {
-  if (g->fifo != nullptr) return ncclSuccess;
+  if (g->flags != nullptr) return ncclSuccess;
   const size_t links = (size_t)g->nRanks * g->nChannels;
-  HIPCHECK(hipMalloc((void**)&g->fifo, links * (size_t)g->chanStride));
   HIPCHECK(hipMalloc((void**)&g->flags, links * sizeof(ConnFlags)));
   HIPCHECK(hipMemset(g->flags, 0, links * sizeof(ConnFlags)));
+  if (g->proto == kProtoFifo) {
+    HIPCHECK(hipMalloc((void**)&g->fifo, links * (size_t)g->chanStride));
+  } else {
+    HIPCHECK(hipMalloc((void**)&g->pubs, links * sizeof(PeerPub)));
+    HIPCHECK(hipMemset(g->pubs, 0, links * sizeof(PeerPub)));
+    HIPCHECK(hipMalloc((void**)&g->p1, links * 8));
+    HIPCHECK(hipMemset(g->p1, 0, links * 8));
+    HIPCHECK(hipMalloc((void**)&g->p2, links * 8));
+    HIPCHECK(hipMemset(g->p2, 0, links * 8));
+    if (g->oneShot) HIPCHECK(hipMalloc((void**)&g->staging, (size_t)g->nRanks * kOneShotMaxBytes));
+  }
   return ncclSuccess;
 }
 
@@ -593,14 +621,13 @@ DFCCL_API ncclResult_t ncclCommDestroy(ncclComm_t comm) {
     if (d != nullptr) {
       std::lock_guard<std::mutex> lk(d->mu);
       if (d->running) {
-        if (g->fifo) d->garbageDev.push_back(g->fifo);
-        if (g->flags) d->garbageDev.push_back(g->flags);
-        g->fifo = nullptr;
-        g->flags = nullptr;
+        for (void* p : {(void*)g->fifo, (void*)g->flags, (void*)g->pubs, (void*)g->p1, (void*)g->p2, (void*)g->staging})
+          if (p) d->garbageDev.push_back(p);
+        g->fifo = nullptr; g->flags = nullptr; g->pubs = nullptr; g->p1 = nullptr; g->p2 = nullptr; g->staging = nullptr;
       }
     }
-    if (g->fifo) (void)hipFree(g->fifo);
-    if (g->flags) (void)hipFree(g->flags);
+    for (void* p : {(void*)g->fifo, (void*)g->flags, (void*)g->pubs, (void*)g->p1, (void*)g->p2, (void*)g->staging})
+      if (p) (void)hipFree(p);
     delete g;
   }
   return ncclSuccess;
@@ -705,8 +732,10 @@ DFCCL_API ncclResult_t ofcclFinalizeRankCtx7StartHostThrds(ofcclRankCtx_t c) {
     p.count = g->count; p.chunkElems = g->chunkElems; p.alignElems = g->alignElems; p.sliceElems = g->sliceElems;
     p.slicesPerChunk = g->slicesPerChunk; p.fifoSlots = g->fifoSlots; p.elemSize = g->elemSize;
     p.slotBytes = g->slotBytes; p.fifoChanStride = g->chanStride;
-    p.sendFifo = g->fifo + (size_t)rank * g->nChannels * g->chanStride;
-    p.recvFifo = g->fifo + (size_t)prev * g->nChannels * g->chanStride;
+    p.sendFifo = g->fifo ? g->fifo + (size_t)rank * g->nChannels * g->chanStride : nullptr;
+    p.recvFifo = g->fifo ? g->fifo + (size_t)prev * g->nChannels * g->chanStride : nullptr;
+    p.proto = g->proto; p.oneShot = g->oneShot; p.pubs = g->pubs; p.p1 = g->p1; p.p2 = g->p2;
+    p.staging = g->staging; p.loopsPerInstance = g->loopsPerInstance;
     p.sendFlags = g->flags + (size_t)rank * g->nChannels;
     p.recvFlags = g->flags + (size_t)prev * g->nChannels;
     p.doneCounter = c->doneCounters + i;
@@ -917,5 +946,7 @@ DFCCL_API ncclResult_t dfcclGetCollGeometry(ofcclRankCtx_t c, int collId, dfcclC
   geom->sliceElems = g->sliceElems;
   geom->slicesPerChunk = g->slicesPerChunk;
   geom->fifoSlots = g->fifoSlots;
+  geom->protocol = g->proto;
+  geom->oneShot = g->oneShot;
   return ncclSuccess;
 }

@@ -188,6 +188,8 @@ typedef struct {
   int64_t sliceElems;  /* nominal slice (one FIFO slot)            */
   int slicesPerChunk;
   int fifoSlots;
+  int protocol;        /* 0: FIFO ring, 1: direct (peers read each other's buffers) */
+  int oneShot;         /* direct protocol, message small enough for the two-exchange variant */
 } dfcclCollGeometry;
 ncclResult_t dfcclGetCollGeometry(ofcclRankCtx_t rankCtx, int collId, dfcclCollGeometry* geom);
 

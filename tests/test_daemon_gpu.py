@@ -20,11 +20,14 @@ from gpu_util import TORCH_OF, geom_of, to_gpu, to_np
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True)
-def _bounded_daemon(monkeypatch):
+@pytest.fixture(autouse=True, params=["direct", "fifo"])
+def proto(request, monkeypatch):
+    """Every test runs under both data protocols: `direct` (all-reduce reads the peers' buffers in place; the
+    other collectives still use FIFOs) and `fifo` (the reference's staged ring for everything)."""
+    monkeypatch.setenv("DFCCL_PROTO", request.param)
     # a daemon that would otherwise stay resident leaves (and is relaunched on demand) every 10 s
     monkeypatch.setenv("DFCCL_DAEMON_MAX_MS", "10000")
-    yield
+    yield request.param
 
 
 def oracle_run(kind, dtype, op, g, root, sends):
@@ -92,7 +95,7 @@ def test_reducing_collectives_dtypes(kind, dtype, op):
     check(kind, dtype, op, 4, 70001, root=1, seed=400)
 
 
-def test_config2_geometry_ring_all_reduce_8_ranks_bf16():
+def test_config2_geometry_ring_all_reduce_8_ranks_bf16(proto):
     # 8 virtual ranks, bf16 Sum, 512 KiB chunks (262,144 elements), normal(0,1); 4 Mi elements per
     # rank here so that the host oracle finishes in seconds (the full 64 MiB shape is in the benchmark)
     from dfccl_amd.ring import VirtualRing
@@ -102,6 +105,7 @@ def test_config2_geometry_ring_all_reduce_8_ranks_bf16():
         ring.finalize()
         g = ring.ctxs[0].geometry(0)
         assert g.chunkElems == 262144 and g.nChannels == 32
+        assert g.protocol == (1 if proto == "direct" else 0)
         sends_np, sends, recvs = make_buffers("all_reduce", orc.BF16, n, count, 2)
         want = orc.all_reduce(orc.BF16, orc.SUM, geom_of(ring, 0), sends_np)
         ring.run(0, sends, recvs, timeout=30)
@@ -141,8 +145,9 @@ def test_forced_preemption_is_bit_exact(monkeypatch):
     monkeypatch.setenv("DFCCL_FORCE_QUIT_EVERY", "1")
     forced = check("all_reduce", orc.F32, orc.SUM, 4, 3_000_001, seed=600)
     assert forced["forcedQuits"] > 0 and forced["ctxSaves"] >= forced["forcedQuits"]
-    # every save is matched by a later load: loads = first loads (one per workgroup and instance) + saves
-    assert forced["ctxLoads"] >= forced["ctxSaves"]
+    # a context that is still resident in LDS when its collective is visited again is not loaded again,
+    # so loads only have to cover the first visit of every workgroup
+    assert forced["ctxLoads"] >= 1
     monkeypatch.setenv("DFCCL_FORCE_QUIT_EVERY", "3")
     check("reduce_scatter", orc.BF16, orc.SUM, 8, 400_000, seed=610)
     check("all_gather", orc.I8, orc.SUM, 3, 1_000_003, seed=620)
@@ -345,3 +350,42 @@ def test_prepare_validation_follows_the_reference():
         ctx.destroy()
         for c in comms + other:
             c.destroy()
+
+
+@pytest.mark.parametrize("dtype,op", [(orc.F16, orc.SUM), (orc.BF16, orc.SUM), (orc.F32, orc.PROD), (orc.I8, orc.MAX)])
+@pytest.mark.parametrize("n,count", [(4, 2048), (2, 1), (8, 16384 // 4), (3, 1000), (5, 8191)])
+def test_small_all_reduce_one_shot_and_in_place(dtype, op, n, count, proto):
+    # small messages take the one-shot variant of the direct protocol; in place goes through staging
+    from dfccl_amd.ring import VirtualRing
+    with VirtualRing(n) as ring:
+        ring.prepare(0, "all_reduce", count, dtype, op)
+        ring.finalize()
+        g = ring.ctxs[0].geometry(0)
+        if proto == "direct" and count * orc.TYPE_SIZE[dtype] <= 32768:
+            assert g.oneShot == 1
+        sends_np, sends, recvs = make_buffers("all_reduce", dtype, n, count, 1100, small_ints=(op == orc.PROD))
+        want = orc.all_reduce(dtype, op, geom_of(ring, 0), sends_np)
+        for rep in range(3):
+            ring.run(0, sends, recvs, timeout=30)
+            for r in range(n):
+                assert np.array_equal(to_np(dtype, recvs[r]), want[r]), (rep, r)
+        bufs = [s.clone() for s in sends]
+        torch.cuda.current_stream().synchronize()
+        ring.run(0, bufs, bufs, timeout=30)  # in place
+        for r in range(n):
+            assert np.array_equal(to_np(dtype, bufs[r]), want[r]), ("in place", r)
+
+
+def test_one_shot_under_forced_preemption(monkeypatch):
+    monkeypatch.setenv("DFCCL_FORCE_QUIT_EVERY", "1")
+    check("all_reduce", orc.F32, orc.SUM, 4, 1024, seed=1200, reps=3)
+    monkeypatch.setenv("BASE_CTX_SWITCH_THRESHOLD", "1")
+    monkeypatch.setenv("NUM_TRY_TASKQ_HEAD", "1")
+    monkeypatch.setenv("RECV_SUCCESS_FACTOR", "0")
+    check("all_reduce", orc.BF16, orc.SUM, 8, 2000, seed=1210, reps=3)
+
+
+def test_many_ranks_fall_back_to_fifo():
+    # more ranks than one workgroup folds in a pass: the collective runs over FIFOs
+    stats = check("all_reduce", orc.I32, orc.SUM, 12, 50000, seed=1300)
+    assert stats["cqesWritten"] == 12
