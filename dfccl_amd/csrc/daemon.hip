@@ -37,6 +37,15 @@ constexpr int kDaemonUnroll = 1;  // see reduce_copy.hip: shallow unrolling keep
 constexpr int kReadyWords = (kMaxColls + 63) / 64;
 enum RunStatus : int { kRunDone = 0, kRunPreempted = 1 };
 
+// Geometry of the direct all-reduce sweeps: loop l covers elements [l * loop, (l + 1) * loop), split into
+// nChannels * n chunks of `real` elements; every loop but the last uses the nominal chunk.
+struct SweepGeom {
+  int64_t count, loop, chunkElems, alignElems;
+  int n, C, ch, es;
+  int me, dtype, op, pad;
+  uint64_t dst;                      // my receive buffer
+  uint64_t peer[kMaxDirectRanks];    // phase 0: the send buffers in fold order; phase 1: the receive buffers by rank
+};
 struct WgShared {
   // scheduler state
   uint64_t frontier;       // next submission ticket this workgroup reads from the mirror ring
@@ -51,6 +60,8 @@ struct WgShared {
   int32_t progressedRound;
   int32_t loadedColl;      // collective whose plan and position are in LDS, -1: none
   int32_t statsDirty;
+  uint32_t traceCount;
+  uint32_t wgIndex;
   // collective being run
   int32_t waitOk;
   int32_t progressed;
@@ -62,6 +73,7 @@ struct WgShared {
   WgStats stats;
   uint64_t peerSend[kMaxDirectRanks];
   uint64_t peerRecv[kMaxDirectRanks];
+  SweepGeom sweep;         // arguments of the direct protocol's sweeps
   uint64_t ready[kReadyWords];
   uint16_t taskq[kMaxColls];
 };
@@ -93,6 +105,15 @@ __device__ __forceinline__ WaitDesc waitFor(const void* ptr, uint64_t value, int
   w.stride = stride;
   w.count = count;
   return w;
+}
+
+// One record of the optional timeline (one thread per workgroup calls this).
+__device__ __forceinline__ void trace(const DaemonArgs& A, WgShared& sh, uint32_t ev, uint32_t arg) {
+  if (A.trace == nullptr) return;
+  const uint32_t i = sh.traceCount++;
+  uint64_t* rec = A.trace + ((size_t)sh.wgIndex * kTraceRecords + (i % kTraceRecords)) * 2;
+  rec[0] = (uint64_t)ev | ((uint64_t)arg << 32);
+  rec[1] = wall_clock64();
 }
 
 // Writes the workgroup's counters to host-coherent memory (thread 0).
@@ -149,6 +170,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
     if (lane == 0) {
       __hip_atomic_store(R.mirrorTail, base + (uint64_t)n, __ATOMIC_RELEASE, DFCCL_AGENT);
       sh.hostFrontier = base + (uint64_t)n;
+      trace(A, sh, kTrSqeFetched, (uint32_t)n);
     }
   }
   // the host may reuse entries every workgroup of the rank has consumed
@@ -164,7 +186,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
 // Wave 0 of every workgroup: take new entries from the mirror ring, one lane per
 // entry, and append the collectives this channel takes part in to the task queue.
 // (Role of checkSQ7TidyTaskQ, enqueue_ofccl_dev.cu:491-627.)
-__device__ __forceinline__ void ingest(const RankDev& R, WgShared& sh, int ch, int lane) {
+__device__ __forceinline__ void ingest(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane) {
   const uint64_t f = sh.frontier;
   const uint64_t tail = __hip_atomic_load(R.mirrorTail, __ATOMIC_ACQUIRE, DFCCL_AGENT);
   const int avail = (int)((tail - f) < 64 ? (tail - f) : 64);
@@ -209,6 +231,7 @@ __device__ __forceinline__ void ingest(const RankDev& R, WgShared& sh, int ch, i
     sh.statsDirty = 1;
     if (added > 0) sh.loadedColl = -1;  // a new instance may have changed the buffers of the cached context
     __hip_atomic_store(&R.wgFrontier[ch], f + (uint64_t)consumed, __ATOMIC_RELAXED, DFCCL_AGENT);
+    trace(A, sh, kTrIngested, (uint32_t)consumed);
   }
 }
 
@@ -249,6 +272,7 @@ __device__ __forceinline__ void waitDescs(const DaemonArgs& A, WgShared& sh, int
                                           const WaitDesc& w1, bool adapt) {
   bool ok;
   int64_t spins = 0;
+  if (lane == 0) trace(A, sh, kTrWaitBegin, (uint32_t)(w0.count + w1.count));
   const int64_t forceEvery = A.knobs.forceQuitEvery;
   if (forceEvery > 0 && sh.slicesSinceLoad >= forceEvery) {
     ok = false;
@@ -270,6 +294,7 @@ __device__ __forceinline__ void waitDescs(const DaemonArgs& A, WgShared& sh, int
     if (ok) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   }
   if (lane == 0) {
+    trace(A, sh, kTrWaitEnd, (uint32_t)((ok ? 1u : 0u) | ((uint32_t)spins << 1)));
     sh.waitOk = ok ? 1 : 0;
     sh.stats.spins += (uint64_t)spins;
     if (ok && adapt) {
@@ -335,60 +360,199 @@ __device__ __forceinline__ void moveSlice(int dtype, int op, const void* s0, con
   }
 }
 
-// Direct protocol: fold n peer buffers (already offset to the chunk) in the order
-// given (n <= kMaxDirectRanks), src[0] first, into dst.  The fold keeps the ring's order for the chunk:
-// src = in[c+1], in[c+2], ..., in[c], each step rounded to the storage type.
-template <int DT, int OP>
-__device__ __forceinline__ void reduceOrdered(const char* const* src, int n, void* dst, size_t nbytes, int tid) {
+// Direct protocol data movement.  A "tile" is one rank's chunk of one loop.
+
+__device__ __forceinline__ uint64_t uniform64(uint64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (uint64_t)lo | ((uint64_t)hi << 32);
+}
+
+// dst[off..] = src[0][off..] (op) src[1][off..] ... (op) src[n-1][off..], folded left to right with every
+// step rounded to the storage type: with src = in[c+1], in[c+2], ..., in[c] this is the ring's order for a
+// chunk owned by rank c.  n <= NS <= kMaxDirectRanks; the NS - n surplus loads re-read src[0] (they hit in
+// cache) so that every array element is defined: predicated loads made the compiler keep the packs in scratch.
+template <int DT, int OP, int NS>
+__device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks], int n, uint64_t dst, int64_t byteOff,
+                                         size_t nbytes, int tid) {
   constexpr int ES = typeSize(DT);
-  uintptr_t align = (uintptr_t)dst;
-  for (int j = 0; j < n; j++) align |= (uintptr_t)src[j];
+  uint64_t align = dst | (uint64_t)byteOff;
+#pragma unroll
+  for (int j = 0; j < NS; j++) align |= src[j];
   size_t doneBytes = 0;
   if ((align & 15u) == 0) {
     const size_t npacks = nbytes >> 4;
+#pragma clang loop vectorize(disable) interleave(disable) unroll(disable)
     for (size_t i = tid; i < npacks; i += kWgThreads) {
-      u32x4 acc;
-      {
-        u32x4 v[8];
+      u32x4 v[NS];
 #pragma unroll
-        for (int j = 0; j < 8; j++)
-          if (j < n) v[j] = loadPack<false>(src[j], i);
-        acc = v[0];
+      for (int j = 0; j < NS; j++) v[j] = loadPack<true>((const char*)(j < n ? src[j] : src[0]) + byteOff, i);
+      u32x4 acc = v[0];
 #pragma unroll
-        for (int j = 1; j < 8; j++)
-          if (j < n) acc = packOp<DT, OP>(acc, v[j]);
-      }
-      storePack<false>(dst, i, acc);
+      for (int j = 1; j < NS; j++)
+        if (j < n) acc = packOp<DT, OP>(acc, v[j]);
+      storePack<false>((char*)dst + byteOff, i, acc);
     }
     doneBytes = npacks << 4;
   }
   const size_t first = doneBytes / ES, nelem = nbytes / ES;
+#pragma clang loop vectorize(disable) interleave(disable) unroll(disable)
   for (size_t i = first + tid; i < nelem; i += kWgThreads) {
-    uint32_t acc = loadElem<ES>(src[0], i);
-    for (int j = 1; j < n; j++) acc = wordOp<DT, OP>(acc, loadElem<ES>(src[j], i));
-    storeElem<ES>(dst, i, acc);
+    uint32_t acc = loadElem<ES>((const char*)src[0] + byteOff, i);
+#pragma unroll
+    for (int j = 1; j < NS; j++)
+      if (j < n) acc = wordOp<DT, OP>(acc, loadElem<ES>((const char*)src[j] + byteOff, i));
+    storeElem<ES>((char*)dst + byteOff, i, acc);
   }
+}
+
+__device__ __forceinline__ int64_t sweepReal(const SweepGeom& g, int64_t l) {
+  const int64_t grid = l * g.loop;
+  if (g.count - grid >= g.loop) return g.chunkElems;
+  return realChunkElems(kAllReduce, g.n, g.C, g.chunkElems, g.alignElems, g.count, grid);
+}
+
+// Phase 0 of the direct all-reduce: for loops [lBegin, lEnd) fold my own chunk from all n send buffers into
+// my receive buffer.  All workgroups sweep the loops together, so at any instant the accesses of the whole
+// grid fall into one window of nChannels * n chunks per buffer.
+template <int DT, int OP, int NS>
+__device__ __forceinline__ void sweepFoldN(const SweepGeom& g, int64_t lBegin, int64_t lEnd, int tid) {
+  for (int64_t l = lBegin; l < lEnd; l++) {
+    const int64_t real = sweepReal(g, l);
+    const int64_t off = l * g.loop + ((int64_t)g.ch * g.n + g.me) * real;
+    const int64_t nelem = (g.count - off < real) ? g.count - off : real;
+    if (nelem > 0) foldTile<DT, OP, NS>(g.peer, g.n, g.dst, off * g.es, (size_t)(nelem * g.es), tid);
+  }
+}
+
+template <int DT, int OP>
+__device__ __forceinline__ void sweepFold(const SweepGeom& g, int64_t lBegin, int64_t lEnd, int tid) {
+  if (g.n <= 2) sweepFoldN<DT, OP, 2>(g, lBegin, lEnd, tid);
+  else if (g.n <= 4) sweepFoldN<DT, OP, 4>(g, lBegin, lEnd, tid);
+  else sweepFoldN<DT, OP, 8>(g, lBegin, lEnd, tid);
 }
 
 template <int DT>
-__device__ __forceinline__ void reduceOrderedOp(int op, const char* const* src, int n, void* dst, size_t nbytes,
-                                                int tid) {
+__device__ __forceinline__ void sweepFoldOp(int op, const SweepGeom& g, int64_t lBegin, int64_t lEnd, int tid) {
   switch (op) {
-    case kSum: reduceOrdered<DT, kSum>(src, n, dst, nbytes, tid); break;
-    case kProd: reduceOrdered<DT, kProd>(src, n, dst, nbytes, tid); break;
-    case kMax: reduceOrdered<DT, kMax>(src, n, dst, nbytes, tid); break;
-    default: reduceOrdered<DT, kMin>(src, n, dst, nbytes, tid); break;
+    case kSum: sweepFold<DT, kSum>(g, lBegin, lEnd, tid); break;
+    case kProd: sweepFold<DT, kProd>(g, lBegin, lEnd, tid); break;
+    case kMax: sweepFold<DT, kMax>(g, lBegin, lEnd, tid); break;
+    default: sweepFold<DT, kMin>(g, lBegin, lEnd, tid); break;
   }
 }
 
-__device__ __forceinline__ void reduceOrderedAny(int dtype, int op, const char* const* src, int n, void* dst,
-                                                 size_t nbytes, int tid) {
+// The geometry and the buffer table are handed over in LDS and copied to registers here.
+__device__ __forceinline__ void sweepFoldAny(const SweepGeom* gp, int64_t lBegin, int64_t lEnd, int tid) {
+  SweepGeom g = *gp;
+#pragma unroll
+  for (int t = 0; t < kMaxDirectRanks; t++) g.peer[t] = uniform64(g.peer[t]);
+  g.dst = uniform64(g.dst);
+  const int op = g.op;
+  switch (g.dtype) {
+    case kF32: sweepFoldOp<kF32>(op, g, lBegin, lEnd, tid); break;
+    case kBF16: sweepFoldOp<kBF16>(op, g, lBegin, lEnd, tid); break;
+    case kF16: sweepFoldOp<kF16>(op, g, lBegin, lEnd, tid); break;
+    case kI32: sweepFoldOp<kI32>(op, g, lBegin, lEnd, tid); break;
+    default: sweepFoldOp<kI8>(op, g, lBegin, lEnd, tid); break;
+  }
+}
+
+// Phase 1: for loops [lBegin, lEnd) copy every peer's chunk from that peer's receive buffer into mine.
+__device__ __forceinline__ void sweepGather(const SweepGeom* gp, int64_t lBegin, int64_t lEnd, int tid) {
+  SweepGeom g = *gp;
+#pragma unroll
+  for (int t = 0; t < kMaxDirectRanks; t++) g.peer[t] = uniform64(g.peer[t]);
+  g.dst = uniform64(g.dst);
+  for (int64_t l = lBegin; l < lEnd; l++) {
+    const int64_t real = sweepReal(g, l);
+    const int64_t chunk0 = l * g.loop + (int64_t)g.ch * g.n * real;
+#pragma unroll
+    for (int j = 0; j < kMaxDirectRanks; j++) {
+      if (j >= g.n || j == g.me) continue;
+      const int64_t off = chunk0 + (int64_t)j * real;
+      const int64_t nelem = (g.count - off < real) ? g.count - off : real;
+      if (nelem <= 0) continue;
+      const void* s[1] = {(const char*)g.peer[j] + off * g.es};
+      void* d[1] = {(char*)g.dst + off * g.es};
+      reduceCopyWG<kI8, kSum, 1, 1, kDaemonUnroll, false>(s, d, (size_t)(nelem * g.es), tid, kWgThreads);
+    }
+  }
+}
+
+// One-shot variant: every rank folds the whole (small) message itself.  The owner of a pack, and with it
+// the fold order, follows from the pack's position; the peers' base pointers are read from LDS.
+template <int DT, int OP, int NS>
+__device__ __forceinline__ void foldOneShotN(const uint64_t* peers, int n, char* out, int64_t count, int64_t real,
+                                             int tid) {
+  constexpr int ES = typeSize(DT);
+  constexpr int PACK = 16 / ES;
+  uint64_t align = (uint64_t)(uintptr_t)out;
+#pragma unroll
+  for (int j = 0; j < NS; j++)
+    if (j < n) align |= peers[j];
+  const int64_t npacks = ((align & 15u) == 0) ? (count / PACK) : 0;
+#pragma clang loop vectorize(disable) interleave(disable) unroll(disable)
+  for (int64_t p = tid; p < npacks; p += kWgThreads) {
+    const int owner = (int)((p * PACK) / real);
+    u32x4 v[NS];
+#pragma unroll
+    for (int t = 0; t < NS; t++) {
+      int idx = owner + 1 + (t < n ? t : 0);
+      if (idx >= n) idx -= n;
+      v[t] = loadPack<false>((const char*)peers[idx], (size_t)p);
+    }
+    u32x4 acc = v[0];
+#pragma unroll
+    for (int t = 1; t < NS; t++)
+      if (t < n) acc = packOp<DT, OP>(acc, v[t]);
+    storePack<false>(out, (size_t)p, acc);
+  }
+#pragma clang loop vectorize(disable) interleave(disable) unroll(disable)
+  for (int64_t i = npacks * PACK + tid; i < count; i += kWgThreads) {
+    const int owner = (int)(i / real);
+    int idx = owner + 1;
+    if (idx >= n) idx -= n;
+    uint32_t acc = loadElem<ES>((const char*)peers[idx], (size_t)i);
+#pragma unroll
+    for (int t = 1; t < NS; t++) {
+      if (t < n) {
+        int k = owner + 1 + t;
+        if (k >= n) k -= n;
+        acc = wordOp<DT, OP>(acc, loadElem<ES>((const char*)peers[k], (size_t)i));
+      }
+    }
+    storeElem<ES>(out, (size_t)i, acc);
+  }
+}
+
+template <int DT, int OP>
+__device__ __forceinline__ void foldOneShot(const uint64_t* peers, int n, char* out, int64_t count, int64_t real,
+                                            int tid) {
+  if (n <= 2) foldOneShotN<DT, OP, 2>(peers, n, out, count, real, tid);
+  else if (n <= 4) foldOneShotN<DT, OP, 4>(peers, n, out, count, real, tid);
+  else foldOneShotN<DT, OP, 8>(peers, n, out, count, real, tid);
+}
+
+template <int DT>
+__device__ __forceinline__ void foldOneShotOp(int op, const uint64_t* peers, int n, char* out, int64_t count,
+                                              int64_t real, int tid) {
+  switch (op) {
+    case kSum: foldOneShot<DT, kSum>(peers, n, out, count, real, tid); break;
+    case kProd: foldOneShot<DT, kProd>(peers, n, out, count, real, tid); break;
+    case kMax: foldOneShot<DT, kMax>(peers, n, out, count, real, tid); break;
+    default: foldOneShot<DT, kMin>(peers, n, out, count, real, tid); break;
+  }
+}
+
+__device__ __forceinline__ void foldOneShotAny(int dtype, int op, const uint64_t* peers, int n, char* out,
+                                               int64_t count, int64_t real, int tid) {
   switch (dtype) {
-    case kF32: reduceOrderedOp<kF32>(op, src, n, dst, nbytes, tid); break;
-    case kBF16: reduceOrderedOp<kBF16>(op, src, n, dst, nbytes, tid); break;
-    case kF16: reduceOrderedOp<kF16>(op, src, n, dst, nbytes, tid); break;
-    case kI32: reduceOrderedOp<kI32>(op, src, n, dst, nbytes, tid); break;
-    default: reduceOrderedOp<kI8>(op, src, n, dst, nbytes, tid); break;
+    case kF32: foldOneShotOp<kF32>(op, peers, n, out, count, real, tid); break;
+    case kBF16: foldOneShotOp<kBF16>(op, peers, n, out, count, real, tid); break;
+    case kF16: foldOneShotOp<kF16>(op, peers, n, out, count, real, tid); break;
+    case kI32: foldOneShotOp<kI32>(op, peers, n, out, count, real, tid); break;
+    default: foldOneShotOp<kI8>(op, peers, n, out, count, real, tid); break;
   }
 }
 
@@ -461,6 +625,7 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
             if (d.send) __hip_atomic_store(&P.sendFlags[ch].tail, sendStep + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
             if (d.recv) __hip_atomic_store(&P.recvFlags[ch].head, recvStep + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
+            trace(A, sh, kTrPosted, (uint32_t)s);
             sh.progressed = 1;
             sh.slicesSinceLoad++;
             sh.stats.slicesMoved++;
@@ -484,23 +649,25 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
 // ----------------------------------------------------------------- direct protocol
 
 // All-reduce in which the virtual ranks read each other's buffers in place.
-// Per loop and channel the n chunks are laid out as in the FIFO ring
-// (ring_schedule.h), chunk j is owned by rank j:
-//   step 0      reduce my own chunk from all n send buffers, in the ring's order
-//               for that chunk, into my receive buffer; then p1[me] = loops done;
-//   step s >= 1 copy chunk j = me - s from rank j's receive buffer once
-//               p1[j] says it is there; after the last one p2[me] = loops done;
-//   finally     wait until every peer's p2 covers the instance: nobody reads my
-//               buffers any more, so the completion may be posted.
-// Messages that fit the registers of one workgroup take a one-shot variant:
-// every rank folds every chunk itself (two flag exchanges in total).
-// Waits are WaitDescs, so every one of them can preempt and resume.
+// Chunks are laid out as in the FIFO ring (ring_schedule.h): loop l, channel c,
+// chunk j (owned by rank j) starts at l * loop + (c * n + j) * real.
+//   publish   my buffers for this instance; wait until every peer has published;
+//   phase 0   sweep all loops: fold my own chunk from the n send buffers, in the
+//             ring's order for that chunk, into my receive buffer; p1[me] = done;
+//   phase 1   wait until every peer's p1 covers the instance, then sweep all loops
+//             again: copy every peer's chunk from its receive buffer; p2[me] = done;
+//   finally   wait until every peer's p2 covers the instance: nobody reads my
+//             buffers any more, so the completion may be posted.
+// Three waits per instance whatever its size; each is a WaitDesc and can preempt.
+// Messages of at most kOneShotMaxBytes on one channel take a one-shot variant:
+// every rank folds every chunk itself (two waits in total).
+// dyn.step is the phase (2 = only the final wait is left), dyn.gridOffset the
+// next loop of the phase, dyn.slice whether the instance is published.
 __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
   const CollPlan& P = sh.plan;
   const int lane = tid & 63, wave = tid >> 6;
   const int n = P.nRanks, C = P.nChannels, es = P.elemSize, me = P.rank;
   const int64_t count = P.count;
-  const int64_t loop = loopElems(kAllReduce, n, C, P.chunkElems);
   const int64_t L = P.loopsPerInstance;
   const uint64_t inst = sh.dyn.instance;
   const uint64_t base = inst * (uint64_t)L;
@@ -508,9 +675,10 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
   const int published = sh.dyn.slice;
   const int peersLoaded = sh.peersLoaded;
   const int pubStride = C * (int)sizeof(PeerPub), ctrStride = C * 8;
+  const int64_t forceEvery = A.knobs.forceQuitEvery;
   PeerPub* myPub = &P.pubs[(size_t)me * C + ch];
-  int64_t grid = sh.dyn.gridOffset;
-  int step0 = sh.dyn.step;
+  int64_t l0 = sh.dyn.gridOffset;
+  int phase = sh.dyn.step;
   __syncthreads();  // every thread has taken its copy of the position before thread 0 changes it
 
   if (!published && tid == 0) {
@@ -536,23 +704,19 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
   }
 
   if (P.oneShot) {
-    // step 0: fold every chunk from the peers' send buffers; step 1: wait until nobody reads any more
+    // phase 0: fold everything; then wait until nobody reads any more (in place: via the staging buffer)
     const int inPlace = (sendbuff == recvbuff);
     char* out = inPlace ? P.staging + (size_t)me * kOneShotMaxBytes : (char*)recvbuff;
-    if (step0 == 0) {
+    if (phase == 0) {
       const int64_t real = realChunkElems(kAllReduce, n, C, P.chunkElems, P.alignElems, count, 0);
-      for (int j = 0; j < n; j++) {
-        const int64_t off = (int64_t)j * real;
-        const int64_t nelem = (count - off < real) ? count - off : real;
-        if (nelem <= 0) break;
-        const char* src[kMaxDirectRanks];
-        for (int t = 0; t < n; t++) src[t] = (const char*)sh.peerSend[(j + 1 + t) % n] + off * es;
-        reduceOrderedAny(P.dtype, P.op, src, n, out + off * es, (size_t)(nelem * es), tid);
-      }
+      if (tid == 0) trace(A, sh, kTrMoveBegin, 0);
+      foldOneShotAny(P.dtype, P.op, sh.peerSend, n, out, count, real, tid);
       __syncthreads();
       if (tid == 0) {
+        trace(A, sh, kTrMoveEnd, 0);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         __hip_atomic_store(&P.p2[(size_t)me * C + ch], base + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
+        trace(A, sh, kTrPosted, 2);
         sh.progressed = 1;
         sh.slicesSinceLoad++;
         sh.stats.slicesMoved++;
@@ -579,69 +743,131 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
     return kRunDone;
   }
 
-  for (; grid < count; grid += loop, step0 = 0) {
-    const int64_t real = realChunkElems(kAllReduce, n, C, P.chunkElems, P.alignElems, count, grid);
-    const uint64_t loopNo = base + (uint64_t)(grid / loop) + 1;
-    const int64_t chunk0 = grid + (int64_t)ch * n * real;
-    for (int s = step0; s < n; ++s) {
-      if (s == 0) {
-        const int64_t off = chunk0 + (int64_t)me * real;
-        const int64_t nelem = (count - off < real) ? count - off : real;
-        if (nelem > 0) {
-          const char* src[kMaxDirectRanks];
-          for (int t = 0; t < n; t++) src[t] = (const char*)sh.peerSend[(me + 1 + t) % n] + off * es;
-          reduceOrderedAny(P.dtype, P.op, src, n, (char*)recvbuff + off * es, (size_t)(nelem * es), tid);
+  if (tid == 0) {
+    SweepGeom& g = sh.sweep;
+    g.count = count;
+    g.loop = loopElems(kAllReduce, n, C, P.chunkElems);
+    g.chunkElems = P.chunkElems;
+    g.alignElems = P.alignElems;
+    g.n = n;
+    g.C = C;
+    g.ch = ch;
+    g.es = es;
+    g.me = me;
+    g.dtype = P.dtype;
+    g.op = P.op;
+    g.pad = 0;
+    g.dst = recvbuff;
+    for (int t = 0; t < kMaxDirectRanks; t++) {
+      if (phase == 0) g.peer[t] = (t < n) ? sh.peerSend[(me + 1 + t) % n] : 0;
+      else g.peer[t] = (t < n) ? sh.peerRecv[t] : 0;
+    }
+  }
+  __syncthreads();
+
+  if (phase == 0) {
+    if (tid == 0) trace(A, sh, kTrMoveBegin, 0);
+    if (forceEvery > 0) {
+      // test hook: one loop at a time, with a preemption point before each
+      for (int64_t l = l0; l < L; l++) {
+        __syncthreads();
+        if (sh.slicesSinceLoad >= forceEvery) {
+          __syncthreads();
+          if (tid == 0) {
+            sh.stats.forcedQuits++;
+            sh.dyn.gridOffset = l;
+            sh.dyn.step = 0;
+          }
+          return kRunPreempted;
         }
         __syncthreads();
+        sweepFoldAny(&sh.sweep, l, l + 1, tid);
         if (tid == 0) {
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-          __hip_atomic_store(&P.p1[(size_t)me * C + ch], loopNo, __ATOMIC_RELAXED, DFCCL_AGENT);
           sh.progressed = 1;
           sh.slicesSinceLoad++;
           sh.stats.slicesMoved++;
         }
-      } else {
-        const int j = (me + n - s) % n;
-        const int64_t off = chunk0 + (int64_t)j * real;
-        const int64_t nelem = (count - off < real) ? count - off : real;
-        if (nelem > 0) {
-          const WaitDesc w0 = waitFor(&P.p1[(size_t)j * C + ch], loopNo, 0, 1);
-          if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
-          __syncthreads();
-          if (!sh.waitOk) {
-            if (tid == 0) {
-              sh.dyn.gridOffset = grid;
-              sh.dyn.step = s;
-            }
-            return kRunPreempted;
-          }
-          copySlice((const char*)sh.peerRecv[j] + off * es, (char*)recvbuff + off * es, nullptr, (size_t)(nelem * es),
-                    tid);
-          if (tid == 0) {
-            sh.progressed = 1;
-            sh.slicesSinceLoad++;
-            sh.stats.slicesMoved++;
-          }
-        }
       }
-      if (s == n - 1) {
-        __syncthreads();
-        if (tid == 0) {
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-          __hip_atomic_store(&P.p2[(size_t)me * C + ch], loopNo, __ATOMIC_RELAXED, DFCCL_AGENT);
-        }
+    } else {
+      sweepFoldAny(&sh.sweep, l0, L, tid);
+      if (tid == 0) {
+        sh.progressed = 1;
+        sh.slicesSinceLoad += L - l0;
+        sh.stats.slicesMoved += (uint64_t)(L - l0);
       }
     }
+    __syncthreads();
+    if (tid == 0) {
+      trace(A, sh, kTrMoveEnd, 0);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      __hip_atomic_store(&P.p1[(size_t)me * C + ch], base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
+      trace(A, sh, kTrPosted, 1);
+      for (int t = 0; t < kMaxDirectRanks; t++) sh.sweep.peer[t] = (t < n) ? sh.peerRecv[t] : 0;
+    }
+    phase = 1;
+    l0 = 0;
   }
-  // nobody may still be reading my send buffer or my chunk of the receive buffer
+
+  if (phase == 1) {
+    const WaitDesc w0 = waitFor(&P.p1[ch], base + (uint64_t)L, ctrStride, n);
+    if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
+    __syncthreads();
+    if (!sh.waitOk) {
+      if (tid == 0) {
+        sh.dyn.gridOffset = l0;
+        sh.dyn.step = 1;
+      }
+      return kRunPreempted;
+    }
+    if (tid == 0) trace(A, sh, kTrMoveBegin, 1);
+    if (forceEvery > 0) {
+      for (int64_t l = l0; l < L; l++) {
+        __syncthreads();
+        if (sh.slicesSinceLoad >= forceEvery) {
+          __syncthreads();
+          if (tid == 0) {
+            sh.stats.forcedQuits++;
+            sh.dyn.gridOffset = l;
+            sh.dyn.step = 1;
+            sh.dyn.wait[0] = noWait();
+            sh.dyn.wait[1] = noWait();
+          }
+          return kRunPreempted;
+        }
+        __syncthreads();
+        sweepGather(&sh.sweep, l, l + 1, tid);
+        if (tid == 0) {
+          sh.progressed = 1;
+          sh.slicesSinceLoad++;
+          sh.stats.slicesMoved++;
+        }
+      }
+    } else {
+      sweepGather(&sh.sweep, l0, L, tid);
+      if (tid == 0) {
+        sh.progressed = 1;
+        sh.slicesSinceLoad += L - l0;
+        sh.stats.slicesMoved += (uint64_t)(L - l0);
+      }
+    }
+    __syncthreads();
+    if (tid == 0) {
+      trace(A, sh, kTrMoveEnd, 1);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      __hip_atomic_store(&P.p2[(size_t)me * C + ch], base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
+      trace(A, sh, kTrPosted, 2);
+    }
+  }
+
+  // nobody may still be reading my send buffer or my chunks of the receive buffer
   {
     const WaitDesc w0 = waitFor(&P.p2[ch], base + (uint64_t)L, ctrStride, n);
     if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
     __syncthreads();
     if (!sh.waitOk) {
       if (tid == 0) {
-        sh.dyn.gridOffset = grid;  // >= count: only this wait is left
-        sh.dyn.step = 0;
+        sh.dyn.gridOffset = 0;
+        sh.dyn.step = 2;
       }
       return kRunPreempted;
     }
@@ -684,6 +910,7 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
     sh.dyn.wait[0] = noWait();
     sh.dyn.wait[1] = noWait();
     sh.statsDirty = 1;
+    trace(A, sh, kTrVisitBegin, coll);
   }
   __syncthreads();
   const int status = runColl(A, sh, ch, tid);
@@ -711,17 +938,19 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
                            cqeEncode((unsigned)ch, (unsigned)(t + 1), (unsigned)sh.plan.collId), __ATOMIC_RELEASE,
                            DFCCL_SYSTEM);
         sh.stats.cqesWritten++;
+        trace(A, sh, kTrCqePosted, coll);
       }
     } else {
       // preempted: save the context (saveExcutingCollCtx, enqueue_ofccl_dev.cu:664-677)
       *dynG = sh.dyn;
       sh.stats.ctxSaves++;
     }
+    trace(A, sh, kTrVisitEnd, (uint32_t)status);
   }
   __syncthreads();
 }
 
-extern "C" __global__ __launch_bounds__(kWgThreads, 4) void dfcclDaemonKernel(const DaemonArgs* __restrict__ argsPtr) {
+extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const DaemonArgs* __restrict__ argsPtr) {
   __shared__ WgShared sh;
   const DaemonArgs& A = *argsPtr;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -748,6 +977,9 @@ extern "C" __global__ __launch_bounds__(kWgThreads, 4) void dfcclDaemonKernel(co
     sh.progressedRound = 0;
     sh.loadedColl = -1;
     sh.peersLoaded = 0;
+    sh.wgIndex = blockIdx.x;
+    sh.traceCount = 0;
+    trace(A, sh, kTrLaunch, A.epoch);
     const WgStats* hs = &R.stats[ch];
     sh.stats.sqesRead = hs->sqesRead;
     sh.stats.cqesWritten = hs->cqesWritten;
@@ -767,7 +999,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads, 4) void dfcclDaemonKernel(co
     // ---- ingest phase (wave 0)
     if (wave == 0) {
       if (ch == 0) pollHost(A, R, sh, lane);
-      ingest(R, sh, ch, lane);
+      ingest(A, R, sh, ch, lane);
       scanReady(R, sh, ch, lane);
       if (lane == 0) {
         const uint32_t abortFlag = __hip_atomic_load(&A.devFlags[1], __ATOMIC_RELAXED, DFCCL_AGENT);
@@ -790,12 +1022,18 @@ extern "C" __global__ __launch_bounds__(kWgThreads, 4) void dfcclDaemonKernel(co
       }
     }
     __syncthreads();
-    if (sh.exitKind != kExitNone) break;
+    // Every thread takes this round's decisions into registers, and only then may wave 0 go on to the next
+    // round and overwrite them (without the second barrier a wave that is late reading numReady could see the
+    // next round's value, enter the run phase alone and leave the workgroup's barriers out of step for good).
+    const int roundExit = sh.exitKind;
+    const int nq = sh.numActive;
+    const int numReady = sh.numReady;
+    __syncthreads();
+    if (roundExit != kExitNone) break;
 
     // ---- run phase: visit the collectives that can move, in arrival order
     // (traverseTaskQ, enqueue_ofccl_dev.cu:922-1016)
-    const int nq = sh.numActive;
-    if (sh.numReady > 0) {
+    if (numReady > 0) {
       for (int wd = 0; wd * 64 < nq; wd++) {
         uint64_t m = sh.ready[wd];
         while (m) {
@@ -830,6 +1068,9 @@ extern "C" __global__ __launch_bounds__(kWgThreads, 4) void dfcclDaemonKernel(co
   }
   __syncthreads();
   if (tid == 0) {
+    trace(A, sh, kTrExit, (uint32_t)exitKind);
+    if (A.trace != nullptr)  // the last record slot of the workgroup holds how many records it wrote
+      A.trace[((size_t)sh.wgIndex * kTraceRecords + (kTraceRecords - 1)) * 2 + 1] = sh.traceCount;
     flushStats(R, sh, ch);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
     __hip_atomic_store(&R.wgExit[ch], (A.epoch << 4) | (uint32_t)exitKind, __ATOMIC_RELEASE, DFCCL_SYSTEM);
@@ -847,3 +1088,4 @@ extern "C" hipError_t dfcclLaunchDaemon(const dfccl::DaemonArgs* devArgs, int nS
   hipLaunchKernelGGL(dfccl::dfcclDaemonKernel, dim3(grid), dim3(dfccl::kWgThreads), 0, stream, devArgs);
   return hipGetLastError();
 }
+

@@ -191,6 +191,15 @@ struct DaemonArgs {
   uint32_t epoch;
   uint32_t pad;
   uint32_t* devFlags;  // HBM: [0] quit request, [1] abort (set by leaders from the control word)
+  // optional timeline (DFCCL_TRACE=1): kTraceRecords records of {event | arg << 32, 100 MHz tick} per workgroup,
+  // the stamps the reference takes under DEBUG_CLOCK (src/include/collectives_ofccl.h:219-299)
+  uint64_t* trace;
+};
+
+constexpr int kTraceRecords = 4096;
+enum TraceEvent : uint32_t {
+  kTrSqeFetched = 1, kTrIngested = 2, kTrVisitBegin = 3, kTrWaitBegin = 4, kTrWaitEnd = 5, kTrMoveBegin = 6,
+  kTrMoveEnd = 7, kTrPosted = 8, kTrCqePosted = 9, kTrVisitEnd = 10, kTrScanDone = 11, kTrLaunch = 12, kTrExit = 13
 };
 
 }  // namespace dfccl

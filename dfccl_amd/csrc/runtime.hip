@@ -13,6 +13,7 @@
 #include <sched.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
@@ -168,13 +169,26 @@ struct Daemon {
   bool failed = false;
   uint32_t epoch = 0;
   uint64_t launches = 0;
+  long capacity = 0;
   uint32_t* ctrl = nullptr;      // host-coherent
   uint32_t* devFlags = nullptr;  // HBM
   DaemonArgs* devArgs = nullptr; // HBM
   DaemonArgs hostArgs{};
+  uint64_t* trace = nullptr;     // HBM, only with DFCCL_TRACE=1
   Knobs knobs{};
   std::thread observer;
   std::vector<void*> garbageDev, garbageHost;
+
+  // Workgroups of the daemon kernel the device can hold at once: all of them must be resident, because a
+  // workgroup that is not resident cannot answer its peers.
+  long residentCapacity() {
+    if (capacity > 0) return capacity;
+    // one 512-thread workgroup of the daemon kernel per CU (it needs more than 128 VGPRs per lane)
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) cus = 0;
+    capacity = (long)cus;
+    return capacity;
+  }
 
   bool wantLaunch() const {
     if (launchRequested) return true;
@@ -217,12 +231,19 @@ struct Daemon {
     if (nSlots == 0) return false;
     // a multiple of 8 channels keeps channel c of every rank on XCD c % 8
     if (chans > 1) chans = (chans + 7) & ~7;
+    if ((long)nSlots * chans > residentCapacity()) {
+      fprintf(stderr,
+              "dfccl: %d rank slots x %d channels do not fit the %ld workgroups the GPU keeps resident; "
+              "lower NCCL_MAX_NCHANNELS\n", nSlots, chans, residentCapacity());
+      return false;
+    }
     epoch++;
     hostArgs.knobs = knobs;
     hostArgs.nSlots = nSlots;
     hostArgs.channelsPerRank = chans;
     hostArgs.epoch = epoch;
     hostArgs.devFlags = devFlags;
+    hostArgs.trace = trace;
     __atomic_store_n(ctrl, 0u, __ATOMIC_RELEASE);
     if (hipMemcpy(devArgs, &hostArgs, sizeof(hostArgs), hipMemcpyHostToDevice) != hipSuccess) return false;
     if (hipMemset(devFlags, 0, 64) != hipSuccess) return false;
@@ -306,6 +327,11 @@ static ncclResult_t getDaemon(int device, Daemon** out) {
   HIPCHECK(hipMalloc((void**)&d->devFlags, 64));
   HIPCHECK(hipMemset(d->devFlags, 0, 64));
   HIPCHECK(hipMalloc((void**)&d->devArgs, sizeof(DaemonArgs)));
+  if (envInt("DFCCL_TRACE", 0) != 0) {
+    const size_t bytes = (size_t)kMaxRankSlots * kMaxChannels * kTraceRecords * 16;
+    HIPCHECK(hipMalloc((void**)&d->trace, bytes));
+    HIPCHECK(hipMemset(d->trace, 0, bytes));
+  }
   d->readKnobs();
   d->observer = std::thread([d] { d->observerLoop(); });
   gDaemons[device] = d;
@@ -336,6 +362,20 @@ static void destroyDaemon(Daemon* d) {
     d->cv.notify_all();
   }
   if (d->observer.joinable()) d->observer.join();
+  if (d->trace != nullptr) {
+    // dump the timeline of the last launch: [workgroup][record]{event | arg << 32, tick}
+    const char* path = getenv("DFCCL_TRACE_FILE");
+    const size_t bytes = (size_t)kMaxRankSlots * kMaxChannels * kTraceRecords * 16;
+    std::vector<char> host(bytes);
+    if (hipMemcpy(host.data(), d->trace, bytes, hipMemcpyDeviceToHost) == hipSuccess) {
+      FILE* f = fopen(path && *path ? path : "dfccl_trace.bin", "wb");
+      if (f) {
+        fwrite(host.data(), 1, bytes, f);
+        fclose(f);
+      }
+    }
+    (void)hipFree(d->trace);
+  }
   d->collectGarbage();
   (void)hipFree(d->devArgs);
   (void)hipFree(d->devFlags);
@@ -363,12 +403,24 @@ static void planGroup(CommGroup* g) {
     g->count = (int64_t)g->countUser;
   }
   if (g->kind == kAllGather || g->kind == kReduceScatter) nBytes *= g->nRanks;
+  // protocol: the virtual ranks of an all-reduce read each other's buffers in place unless told otherwise
+  const char* proto = getenv("DFCCL_PROTO");
+  const bool wantFifo = proto != nullptr && strcmp(proto, "fifo") == 0;
+  g->proto = (!wantFifo && g->kind == kAllReduce && g->nRanks >= 2 && g->nRanks <= kMaxDirectRanks) ? kProtoDirect
+                                                                                                     : kProtoFifo;
   int64_t buff = envInt("NCCL_BUFFSIZE", 1 << 20);
   if (buff < (64 << 10)) buff = 64 << 10;
   buff = (buff / (8 * kAlignBytes)) * (8 * kAlignBytes);
   const int64_t stepBytes = buff / 8;  // NCCL_STEPS = 8
   int64_t chunkBytes, sliceBytes;
-  if (g->kind == kReduce || g->kind == kBroadcast) {  // CHUNKSTEPS = SLICESTEPS = 1
+  if (g->proto == kProtoDirect) {
+    // no FIFO: the chunk is only the interleaving grain of the sweeps (small grains keep all workgroups
+    // inside one compact address window per buffer)
+    chunkBytes = roundUp64(std::max<int64_t>(envInt("DFCCL_DIRECT_CHUNK_BYTES", 16 << 10), kAlignBytes), kAlignBytes);
+    sliceBytes = chunkBytes;
+    g->slicesPerChunk = 1;
+    g->fifoSlots = 1;
+  } else if (g->kind == kReduce || g->kind == kBroadcast) {  // CHUNKSTEPS = SLICESTEPS = 1
     chunkBytes = stepBytes;
     sliceBytes = stepBytes;
     g->slicesPerChunk = 1;
@@ -393,11 +445,6 @@ static void planGroup(CommGroup* g) {
   const int64_t maxSlice = sliceElemsFor(real0, g->slicesPerChunk, g->sliceElems);
   g->slotBytes = roundUp64(maxSlice * g->elemSize, kAlignBytes);
   g->chanStride = g->slotBytes * g->fifoSlots;
-  // protocol: the virtual ranks of an all-reduce read each other's buffers in place unless told otherwise
-  const char* proto = getenv("DFCCL_PROTO");
-  const bool wantFifo = proto != nullptr && strcmp(proto, "fifo") == 0;
-  g->proto = (!wantFifo && g->kind == kAllReduce && g->nRanks >= 2 && g->nRanks <= kMaxDirectRanks) ? kProtoDirect
-                                                                                                   : kProtoFifo;
   const int64_t loop = loopElems(g->kind, g->nRanks, g->nChannels, g->chunkElems);
   g->loopsPerInstance = g->count > 0 ? divUp64(g->count, loop) : 0;
   g->oneShot = (g->proto == kProtoDirect && g->nChannels == 1 && g->loopsPerInstance <= 1 &&

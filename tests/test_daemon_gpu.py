@@ -95,17 +95,22 @@ def test_reducing_collectives_dtypes(kind, dtype, op):
     check(kind, dtype, op, 4, 70001, root=1, seed=400)
 
 
-def test_config2_geometry_ring_all_reduce_8_ranks_bf16(proto):
+@pytest.mark.parametrize("chunk_bytes", [524288, None])
+def test_config2_geometry_ring_all_reduce_8_ranks_bf16(proto, chunk_bytes, monkeypatch):
     # 8 virtual ranks, bf16 Sum, 512 KiB chunks (262,144 elements), normal(0,1); 4 Mi elements per
-    # rank here so that the host oracle finishes in seconds (the full 64 MiB shape is in the benchmark)
+    # rank here so that the host oracle finishes in seconds (the full 64 MiB shape is in the benchmark).
+    # chunk_bytes None: the library's own grain for the direct protocol (the FIFO default is 512 KiB).
     from dfccl_amd.ring import VirtualRing
     n, count = 8, 4 << 20
+    if chunk_bytes is not None:
+        monkeypatch.setenv("DFCCL_DIRECT_CHUNK_BYTES", str(chunk_bytes))
     with VirtualRing(n) as ring:
         ring.prepare(0, "all_reduce", count, orc.BF16, orc.SUM)
         ring.finalize()
         g = ring.ctxs[0].geometry(0)
-        assert g.chunkElems == 262144 and g.nChannels == 32
-        assert g.protocol == (1 if proto == "direct" else 0)
+        assert g.nChannels == 32 and g.protocol == (1 if proto == "direct" else 0)
+        if chunk_bytes is not None or proto == "fifo":
+            assert g.chunkElems == 262144
         sends_np, sends, recvs = make_buffers("all_reduce", orc.BF16, n, count, 2)
         want = orc.all_reduce(orc.BF16, orc.SUM, geom_of(ring, 0), sends_np)
         ring.run(0, sends, recvs, timeout=30)
