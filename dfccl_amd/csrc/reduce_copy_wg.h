@@ -13,15 +13,18 @@
 
 namespace dfccl {
 
+// All operands of the data path are in global memory (HBM or host-coherent), never LDS or scratch: saying so
+// turns what would be flat_load / flat_store (pointers that come out of context structures have no known
+// address space) into global_load / global_store, which do not also occupy the LDS path.
 template <bool NT>
 __device__ __forceinline__ u32x4 loadPack(const void* base, size_t pack) {
-  const u32x4* p = (const u32x4*)base + pack;
+  const DFCCL_GLOBAL u32x4* p = (const DFCCL_GLOBAL u32x4*)base + pack;
   if constexpr (NT) return __builtin_nontemporal_load(p);
   else return *p;
 }
 template <bool NT>
 __device__ __forceinline__ void storePack(void* base, size_t pack, u32x4 v) {
-  u32x4* p = (u32x4*)base + pack;
+  DFCCL_GLOBAL u32x4* p = (DFCCL_GLOBAL u32x4*)base + pack;
   if constexpr (NT) __builtin_nontemporal_store(v, p);
   else *p = v;
 }

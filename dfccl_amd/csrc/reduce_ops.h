@@ -98,18 +98,20 @@ __device__ __forceinline__ u32x4 packOp(u32x4 a, u32x4 b) {
   return r;
 }
 
-// One element held in the low bits of a word (upper bits zero).
+#define DFCCL_GLOBAL __attribute__((address_space(1)))
+
+// One element held in the low bits of a word (upper bits zero). Operands are in global memory.
 template <int ES>
 __device__ __forceinline__ uint32_t loadElem(const void* p, size_t i) {
-  if constexpr (ES == 1) return ((const uint8_t*)p)[i];
-  else if constexpr (ES == 2) return ((const uint16_t*)p)[i];
-  else return ((const uint32_t*)p)[i];
+  if constexpr (ES == 1) return ((const DFCCL_GLOBAL uint8_t*)p)[i];
+  else if constexpr (ES == 2) return ((const DFCCL_GLOBAL uint16_t*)p)[i];
+  else return ((const DFCCL_GLOBAL uint32_t*)p)[i];
 }
 template <int ES>
 __device__ __forceinline__ void storeElem(void* p, size_t i, uint32_t v) {
-  if constexpr (ES == 1) ((uint8_t*)p)[i] = (uint8_t)v;
-  else if constexpr (ES == 2) ((uint16_t*)p)[i] = (uint16_t)v;
-  else ((uint32_t*)p)[i] = v;
+  if constexpr (ES == 1) ((DFCCL_GLOBAL uint8_t*)p)[i] = (uint8_t)v;
+  else if constexpr (ES == 2) ((DFCCL_GLOBAL uint16_t*)p)[i] = (uint16_t)v;
+  else ((DFCCL_GLOBAL uint32_t*)p)[i] = v;
 }
 
 }  // namespace dfccl
