@@ -62,6 +62,9 @@ struct WgShared {
   int32_t statsDirty;
   uint32_t traceCount;
   uint32_t wgIndex;
+  uint32_t round;          // scheduler rounds since launch
+  int32_t allFresh;        // every collective of the task queue was ingested this round (nothing is parked)
+  uint64_t cqNext;         // single-channel ranks: next completion ticket
   // collective being run
   int32_t waitOk;
   int32_t progressed;
@@ -76,6 +79,7 @@ struct WgShared {
   SweepGeom sweep;         // arguments of the direct protocol's sweeps
   uint64_t ready[kReadyWords];
   uint16_t taskq[kMaxColls];
+  uint8_t collChannels[kMaxColls];  // channels of every collective of this rank (copied from the plans at launch)
 };
 
 #define DFCCL_AGENT __HIP_MEMORY_SCOPE_AGENT
@@ -130,8 +134,51 @@ __device__ __forceinline__ void flushStats(const RankDev& R, WgShared& sh, int c
   sh.statsDirty = 0;
 }
 
-// Leader, wave 0: fetch submissions from the host ring into the HBM mirror and
-// pick up the host's control word.  (Role of sqRead, enqueue_ofccl_dev.cu:85-173.)
+// Wave 0: append the entries held one per lane (lanes < avail) to the task queue if this channel takes part
+// in them; a quit entry ends the batch.  (Role of checkSQ7TidyTaskQ, enqueue_ofccl_dev.cu:491-627.)
+__device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane,
+                                              int avail, uint64_t sendbuff, uint64_t recvbuff, uint32_t coll,
+                                              uint32_t flags) {
+  // buffers named by the new entries may have been written by the host, a copy engine or another kernel
+  // before the submission
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+  bool isQuit = false, mine = false;
+  if (lane < avail) {
+    isQuit = (flags & kSqeFlagQuit) != 0;
+    if (!isQuit && coll < (uint32_t)R.nColls) mine = ch < (int)sh.collChannels[coll];
+  }
+  const uint64_t qm = __ballot(isQuit);
+  const int q = qm ? (int)__builtin_ctzll(qm) : 64;
+  const int take = avail < q ? avail : q;
+  const uint64_t mm = __ballot(mine && lane < take);
+  const int pos = __builtin_popcountll(mm & ((1ull << lane) - 1ull));
+  const int base = sh.numActive;
+  if (mine && lane < take && base + pos < kMaxColls) {
+    DynCtx* d = &R.dyn[(size_t)ch * R.nColls + coll];
+    d->sendbuff = sendbuff;
+    d->recvbuff = recvbuff;
+    d->active = 1;
+    sh.taskq[base + pos] = (uint16_t)coll;
+  }
+  if (lane == 0) {
+    const int added = __builtin_popcountll(mm);
+    sh.numActive = base + added;
+    const int consumed = take + (q < avail ? 1 : 0);
+    sh.frontier += (uint64_t)consumed;
+    if (q < avail) sh.finalQuit = 1;
+    sh.ingested = consumed;
+    sh.allFresh = (base == 0) ? 1 : 0;
+    sh.stats.sqesRead += (uint64_t)consumed;
+    sh.statsDirty = 1;
+    if (added > 0) sh.loadedColl = -1;  // a new instance may have changed the buffers of the cached context
+    if (R.nChannels > 1) __hip_atomic_store(&R.wgFrontier[ch], sh.frontier, __ATOMIC_RELAXED, DFCCL_AGENT);
+    trace(A, sh, kTrIngested, (uint32_t)consumed);
+  }
+}
+
+// Leader, wave 0: fetch submissions from the host ring (four lanes per entry, each word validated by its own
+// tag), hand them to the other channels through the HBM mirror, take them into the own task queue straight
+// from the registers, and pick up the host's control word.  (Role of sqRead, enqueue_ofccl_dev.cu:85-173.)
 __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, WgShared& sh, int lane) {
   const uint64_t base = sh.hostFrontier;
   uint64_t w = 0;
@@ -152,41 +199,54 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
   const uint64_t vm = __ballot(valid);
   int n = 0;
   while (n < kSqesPerPoll && ((vm >> (4 * n)) & 0xfull) == 0xfull) n++;
-  if (n > 0) {
-    const int first = lane & ~3;
-    const uint64_t w1 = __shfl(w, first + 1);
-    const uint64_t w2 = __shfl(w, first + 2);
-    if ((lane & 3) == 0 && (lane >> 2) < n) {
-      const uint64_t ticket = base + (uint64_t)(lane >> 2);
-      DevSqe* e = &R.mirror[ticket & (kSqRing - 1)];
-      e->sendbuff = w & kPtrMask;
-      e->recvbuff = w1 & kPtrMask;
-      e->coll = (uint32_t)(w2 & 0xffffffffull);
-      e->flags = (uint32_t)((w2 >> 32) & 0xffffull);
-      e->ticket = ticket;
+  if (n == 0) {
+    if (lane == 0) sh.ingested = 0;
+  } else {
+    // lane k < n takes entry k
+    const int srcLane = (lane * 4) & 63;
+    const uint64_t w0 = __shfl(w, srcLane);
+    const uint64_t w1 = __shfl(w, srcLane + 1);
+    const uint64_t w2 = __shfl(w, srcLane + 2);
+    const uint64_t sendbuff = w0 & kPtrMask, recvbuff = w1 & kPtrMask;
+    const uint32_t coll = (uint32_t)(w2 & 0xffffffffull), flags = (uint32_t)((w2 >> 32) & 0xffffull);
+    if (R.nChannels > 1) {
+      if (lane < n) {
+        const uint64_t ticket = base + (uint64_t)lane;
+        DevSqe* e = &R.mirror[ticket & (kSqRing - 1)];
+        e->sendbuff = sendbuff;
+        e->recvbuff = recvbuff;
+        e->coll = coll;
+        e->flags = flags;
+        e->ticket = ticket;
+      }
+      // every lane's entry is written before lane 0 publishes the new tail
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      if (lane == 0) __hip_atomic_store(R.mirrorTail, base + (uint64_t)n, __ATOMIC_RELAXED, DFCCL_AGENT);
     }
-    // every lane's entry is written before lane 0 publishes the new tail
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     if (lane == 0) {
-      __hip_atomic_store(R.mirrorTail, base + (uint64_t)n, __ATOMIC_RELEASE, DFCCL_AGENT);
       sh.hostFrontier = base + (uint64_t)n;
       trace(A, sh, kTrSqeFetched, (uint32_t)n);
     }
+    ingestEntries(A, R, sh, 0, lane, n, sendbuff, recvbuff, coll, flags);
   }
-  // the host may reuse entries every workgroup of the rank has consumed
-  uint64_t f = ~0ull;
-  if (lane < R.nChannels) f = __hip_atomic_load(&R.wgFrontier[lane], __ATOMIC_RELAXED, DFCCL_AGENT);
-  f = waveMin64(f);
-  if (lane == 0 && f != sh.publishedHead) {
-    __hip_atomic_store(R.sqHead, f, __ATOMIC_RELAXED, DFCCL_SYSTEM);
-    sh.publishedHead = f;
+  // The host may reuse entries every workgroup of the rank has consumed. It only looks at the head when the
+  // ring seems full, so the head is published now and then, not on every poll.
+  if (sh.hostFrontier - sh.publishedHead >= 64 || (n == 0 && sh.hostFrontier != sh.publishedHead)) {
+    uint64_t f = sh.frontier;
+    if (R.nChannels > 1) {
+      f = ~0ull;
+      if (lane < R.nChannels) f = __hip_atomic_load(&R.wgFrontier[lane], __ATOMIC_RELAXED, DFCCL_AGENT);
+      f = waveMin64(f);
+    }
+    if (lane == 0 && f != sh.publishedHead) {
+      __hip_atomic_store(R.sqHead, f, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+      sh.publishedHead = f;
+    }
   }
 }
 
-// Wave 0 of every workgroup: take new entries from the mirror ring, one lane per
-// entry, and append the collectives this channel takes part in to the task queue.
-// (Role of checkSQ7TidyTaskQ, enqueue_ofccl_dev.cu:491-627.)
-__device__ __forceinline__ void ingest(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane) {
+// Wave 0 of the other channels: take new entries from the mirror ring, one lane per entry.
+__device__ __forceinline__ void ingestMirror(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane) {
   const uint64_t f = sh.frontier;
   const uint64_t tail = __hip_atomic_load(R.mirrorTail, __ATOMIC_ACQUIRE, DFCCL_AGENT);
   const int avail = (int)((tail - f) < 64 ? (tail - f) : 64);
@@ -194,45 +254,12 @@ __device__ __forceinline__ void ingest(const DaemonArgs& A, const RankDev& R, Wg
     if (lane == 0) sh.ingested = 0;
     return;
   }
-  // buffers named by the new entries may have been written by the host, a copy
-  // engine or another kernel before the submission
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
   DevSqe e;
   e.sendbuff = e.recvbuff = 0;
   e.coll = 0;
   e.flags = 0;
-  bool isQuit = false, mine = false;
-  if (lane < avail) {
-    e = R.mirror[(f + (uint64_t)lane) & (kSqRing - 1)];
-    isQuit = (e.flags & kSqeFlagQuit) != 0;
-    if (!isQuit && e.coll < (uint32_t)R.nColls) mine = ch < R.plans[e.coll].nChannels;
-  }
-  const uint64_t qm = __ballot(isQuit);
-  const int q = qm ? (int)__builtin_ctzll(qm) : 64;
-  const int take = avail < q ? avail : q;
-  const uint64_t mm = __ballot(mine && lane < take);
-  const int pos = __builtin_popcountll(mm & ((1ull << lane) - 1ull));
-  const int base = sh.numActive;
-  if (mine && lane < take && base + pos < kMaxColls) {
-    DynCtx* d = &R.dyn[(size_t)ch * R.nColls + e.coll];
-    d->sendbuff = e.sendbuff;
-    d->recvbuff = e.recvbuff;
-    d->active = 1;
-    sh.taskq[base + pos] = (uint16_t)e.coll;
-  }
-  if (lane == 0) {
-    const int added = __builtin_popcountll(mm);
-    sh.numActive = base + added;
-    const int consumed = take + (q < avail ? 1 : 0);
-    sh.frontier = f + (uint64_t)consumed;
-    if (q < avail) sh.finalQuit = 1;
-    sh.ingested = consumed;
-    sh.stats.sqesRead += (uint64_t)consumed;
-    sh.statsDirty = 1;
-    if (added > 0) sh.loadedColl = -1;  // a new instance may have changed the buffers of the cached context
-    __hip_atomic_store(&R.wgFrontier[ch], f + (uint64_t)consumed, __ATOMIC_RELAXED, DFCCL_AGENT);
-    trace(A, sh, kTrIngested, (uint32_t)consumed);
-  }
+  if (lane < avail) e = R.mirror[(f + (uint64_t)lane) & (kSqRing - 1)];
+  ingestEntries(A, R, sh, ch, lane, avail, e.sendbuff, e.recvbuff, e.coll, e.flags);
 }
 
 // One lane: is this parked collective's wait condition met?
@@ -249,6 +276,14 @@ __device__ __forceinline__ bool descMet(const WaitDesc& w) {
 __device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, int ch, int lane) {
   const int n = sh.numActive;
   int total = 0;
+  if (sh.allFresh && sh.ingested > 0 && n <= 64) {
+    // nothing is parked: everything in the queue arrived this round and can start
+    if (lane == 0) {
+      sh.ready[0] = (n >= 64) ? ~0ull : ((1ull << n) - 1ull);
+      sh.numReady = n;
+    }
+    return;
+  }
   for (int base = 0; base < n; base += 64) {
     const int i = base + lane;
     bool ready = false;
@@ -926,20 +961,26 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
       if (sh.plan.proto == kProtoFifo) sh.dyn.slice = 0;
       sh.dyn.wait[0] = noWait();
       sh.dyn.wait[1] = noWait();
-      *dynG = sh.dyn;
       sh.taskq[qi] = (uint16_t)kInvalidTask;
-      // completion (manipulateCQ7ResetDoneColl, enqueue_ofccl_dev.cu:773-920): the last
-      // channel to finish posts the entry; results are released to the system first
+      // completion (manipulateCQ7ResetDoneColl, enqueue_ofccl_dev.cu:773-920): results are released to the
+      // system, then the last channel to finish posts the entry
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-      const uint64_t old = __hip_atomic_fetch_add(sh.plan.doneCounter, 1ull, __ATOMIC_ACQ_REL, DFCCL_AGENT);
-      if ((old + 1) % (uint64_t)sh.plan.nChannels == 0) {
-        const uint64_t t = __hip_atomic_fetch_add(R.cqTicket, 1ull, __ATOMIC_RELAXED, DFCCL_AGENT);
+      bool last = true;
+      if (sh.plan.nChannels > 1) {
+        const uint64_t old = __hip_atomic_fetch_add(sh.plan.doneCounter, 1ull, __ATOMIC_ACQ_REL, DFCCL_AGENT);
+        last = ((old + 1) % (uint64_t)sh.plan.nChannels == 0);
+      }
+      if (last) {
+        // a rank with a single channel has a single poster, which keeps the ticket itself
+        const uint64_t t = (R.nChannels == 1) ? sh.cqNext++
+                                              : __hip_atomic_fetch_add(R.cqTicket, 1ull, __ATOMIC_RELAXED, DFCCL_AGENT);
         __hip_atomic_store(&R.cq[t & (kCqRing - 1)],
                            cqeEncode((unsigned)ch, (unsigned)(t + 1), (unsigned)sh.plan.collId), __ATOMIC_RELEASE,
                            DFCCL_SYSTEM);
         sh.stats.cqesWritten++;
         trace(A, sh, kTrCqePosted, coll);
       }
+      *dynG = sh.dyn;
     } else {
       // preempted: save the context (saveExcutingCollCtx, enqueue_ofccl_dev.cu:664-677)
       *dynG = sh.dyn;
@@ -979,6 +1020,9 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     sh.peersLoaded = 0;
     sh.wgIndex = blockIdx.x;
     sh.traceCount = 0;
+    sh.round = 0;
+    sh.allFresh = 0;
+    sh.cqNext = S.cqNext;
     trace(A, sh, kTrLaunch, A.epoch);
     const WgStats* hs = &R.stats[ch];
     sh.stats.sqesRead = hs->sqesRead;
@@ -993,18 +1037,25 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
   }
   __syncthreads();
   for (int i = tid; i < sh.numActive; i += kWgThreads) sh.taskq[i] = S.taskq[i];
+  for (int i = tid; i < R.nColls; i += kWgThreads) sh.collChannels[i] = (uint8_t)R.plans[i].nChannels;
   __syncthreads();
 
   for (;;) {
     // ---- ingest phase (wave 0)
     if (wave == 0) {
       if (ch == 0) pollHost(A, R, sh, lane);
-      ingest(A, R, sh, ch, lane);
-      scanReady(R, sh, ch, lane);
+      else ingestMirror(A, R, sh, ch, lane);
+      if (sh.numActive > 0) scanReady(R, sh, ch, lane);
+      else if (lane == 0) sh.numReady = 0;
       if (lane == 0) {
-        const uint32_t abortFlag = __hip_atomic_load(&A.devFlags[1], __ATOMIC_RELAXED, DFCCL_AGENT);
-        const uint32_t quitFlag = __hip_atomic_load(&A.devFlags[0], __ATOMIC_RELAXED, DFCCL_AGENT);
-        const bool expired = K.maxLifetimeTicks > 0 && (int64_t)(wall_clock64() - startTick) > K.maxLifetimeTicks;
+        // the host's requests and the lifetime limit are looked at every 8th round: nobody waits on them
+        uint32_t abortFlag = 0, quitFlag = 0;
+        bool expired = false;
+        if ((sh.round++ & 7u) == 0) {
+          abortFlag = __hip_atomic_load(&A.devFlags[1], __ATOMIC_RELAXED, DFCCL_AGENT);
+          quitFlag = __hip_atomic_load(&A.devFlags[0], __ATOMIC_RELAXED, DFCCL_AGENT);
+          expired = K.maxLifetimeTicks > 0 && (int64_t)(wall_clock64() - startTick) > K.maxLifetimeTicks;
+        }
         if (sh.ingested > 0 || sh.progressedRound) sh.idle = 0;
         else sh.idle++;
         if (abortFlag) sh.exitKind = kExitAbort;
@@ -1017,8 +1068,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
       }
       if (sh.numReady == 0 && sh.ingested == 0) {
         // nothing can move: the leader's next poll is a PCIe round trip anyway, the others back off a little
-        if (ch == 0) __builtin_amdgcn_s_sleep(2);
-        else __builtin_amdgcn_s_sleep(20);
+        if (ch != 0) __builtin_amdgcn_s_sleep(20);
       }
     }
     __syncthreads();
@@ -1063,6 +1113,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
       S.frontier = sh.frontier;
       S.hostFrontier = sh.hostFrontier;
       S.numActive = sh.numActive;
+      S.cqNext = sh.cqNext;
       sh.stats.voluntaryQuits++;
     }
   }

@@ -146,6 +146,7 @@ struct WgSaved {
   uint64_t hostFrontier;  // leader only: next host-ring ticket to read
   int32_t numActive;
   int32_t finalQuit;
+  uint64_t cqNext;        // single-channel ranks: next completion ticket (kept by the one workgroup that posts)
   uint16_t taskq[kMaxColls];
 };
 

@@ -882,8 +882,8 @@ DFCCL_API ncclResult_t ofcclDestroy(ofcclRankCtx_t c) {
       }
       if (!quitSent) {
         lk.unlock();
-        // the quit entry (src/enqueue_ofccl.cc:1593-1594)
-        c->submitted.fetch_add(1, std::memory_order_acq_rel);
+        // the quit entry (src/enqueue_ofccl.cc:1593-1594). It does not count as outstanding work: if the
+        // kernel ends before reading it, the rank is simply left out of the next launch.
         while (sqWrite(c, 0, 0, 0, kSqeFlagQuit) == -1) sched_yield();
         quitSent = true;
         continue;
