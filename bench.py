@@ -9,8 +9,10 @@ figure feeds the `roofline` object (bound: HBM, peak 8 TB/s).
 
 Also reported on the same line: the CPU oracle's reduce-copy timed on this
 host's cores (`cpu_baseline`, a bounded sample), the 8-virtual-rank bf16 ring
-all-reduce through the daemon kernel (64 MiB per rank), and the
-submission-to-completion latency of 4 KiB all-reduces.
+all-reduce through the daemon kernel (64 MiB per rank), the
+submission-to-completion latency of 4 KiB all-reduces, the disordered
+small-collective workload and the gradient-bucket workload (all four through
+the native driver dfccl_amd/dfccl_bench, one host thread per virtual rank).
 """
 import argparse
 import json
@@ -81,67 +83,69 @@ def bench_cpu_baseline(budget_s=12.0, nbytes=256 << 20):
                        f"{out['all'][1]} threads; single thread: {out['single'][0]:.2f} GB/s")}
 
 
-def bench_daemon_all_reduce(iters=6, n=8, nbytes=64 << 20):
-    """Config: ring all-reduce over 8 virtual ranks, bf16 Sum, 64 MiB per rank, through the daemon."""
-    import torch
-    import dfccl_amd
-    from dfccl_amd.ring import VirtualRing
-    count = nbytes // 2
-    g = torch.Generator(device="cuda:0").manual_seed(2)
-    sends = [torch.randn(count, device="cuda:0", generator=g).to(torch.bfloat16) for _ in range(n)]
-    recvs = [torch.empty_like(s) for s in sends]
-    torch.cuda.current_stream().synchronize()
-    times = []
-    with VirtualRing(n) as ring:
-        ring.prepare(0, "all_reduce", count, dfccl_amd.ncclBfloat16, dfccl_amd.ncclSum)
-        ring.finalize()
-        geom = ring.ctxs[0].geometry(0)
-        for i in range(iters + 2):
-            t0 = time.perf_counter()
-            ring.run(0, sends, recvs, timeout=60)
-            dt = time.perf_counter() - t0
-            if i >= 2:
-                times.append(dt)
-        stats = ring.stats()
-    ref = sends[0].float()
-    for s in sends[1:]:
-        ref = ref + s.float()
-    err = (recvs[0].float() - ref).abs().max().item()
-    same = all(torch.equal(recvs[0], r) for r in recvs[1:])
-    best = min(times)
-    # bytes the ring schedule moves: per rank (6n-4)/n * N * s (FIFO write and read counted)
-    sched_bytes = (6 * n - 4) / n * nbytes * n
-    return {"workload": f"ring all-reduce, {n} virtual ranks x {nbytes >> 20} MiB bf16 Sum, "
-                        f"{geom.chunkElems * 2 >> 10} KiB chunks, {geom.nChannels} channels/rank",
-            "ms": round(best * 1e3, 3), "algbw_GBps": round(nbytes / best / 1e9, 1),
-            "busbw_GBps": round(nbytes / best / 1e9 * 2 * (n - 1) / n, 1),
-            "schedule_GBps": round(sched_bytes / best / 1e9, 1),
-            "frac_of_hbm_peak": round(sched_bytes / best / 1e9 / HBM_PEAK_GBPS, 4),
-            "ranks_agree": same, "max_abs_err_vs_fp32_sum": err, "ctx_saves": stats["ctxSaves"]}
+NATIVE_DRIVER = os.path.join(ROOT, "dfccl_amd", "dfccl_bench")
 
 
-def bench_latency(n=4, count=2048, iters=300):
-    """Submission-to-completion time of 4 KiB fp16 all-reduces over 4 virtual ranks, measured around the
-    Python submit / callback pair of the last-submitting rank (includes ctypes overhead)."""
-    import torch
-    import dfccl_amd
-    from dfccl_amd.ring import VirtualRing
-    sends = [torch.ones(count, device="cuda:0", dtype=torch.float16) for _ in range(n)]
-    recvs = [torch.empty_like(s) for s in sends]
-    torch.cuda.current_stream().synchronize()
-    lat = []
-    with VirtualRing(n) as ring:
-        ring.prepare(0, "all_reduce", count, dfccl_amd.ncclFloat16, dfccl_amd.ncclSum)
-        ring.finalize()
-        for i in range(iters + 20):
-            ring.run(0, sends, recvs, timeout=30)
-            if i >= 20:
-                last = (n - 1, 0)
-                lat.append((ring.t_done[last] - ring.t_submit[last]) * 1e6)
-    lat.sort()
-    return {"workload": f"{n} virtual ranks, {count * 2} B fp16 all-reduce, last submitter's submit->callback",
-            "p50_us": round(lat[len(lat) // 2], 2), "p90_us": round(lat[int(len(lat) * 0.9)], 2),
-            "p99_us": round(lat[int(len(lat) * 0.99)], 2), "min_us": round(lat[0], 2)}
+def run_native(args, env=None, timeout=180):
+    """Runs one mode of the native driver (dfccl_amd/csrc/bench/dfccl_bench.cc: one host thread per virtual rank,
+    public C ABI only) and returns its JSON object."""
+    import subprocess
+    if not os.path.exists(NATIVE_DRIVER):
+        raise RuntimeError(f"{NATIVE_DRIVER} is missing: run __graft_entry__.build()")
+    e = dict(os.environ)
+    e.setdefault("DFCCL_DAEMON_MAX_MS", "20000")
+    if env:
+        e.update(env)
+    out = subprocess.run([NATIVE_DRIVER] + [str(a) for a in args], env=e, capture_output=True, text=True,
+                         timeout=timeout)
+    if out.returncode != 0:
+        raise RuntimeError(f"dfccl_bench {args} failed: {out.stderr[-500:]}")
+    return json.loads(out.stdout.strip().splitlines()[-1])
+
+
+def bench_daemon_all_reduce():
+    """Ring all-reduce over 8 virtual ranks, bf16 Sum, 64 MiB per rank, through the daemon kernel: once with
+    the library's defaults (direct protocol, 16 KiB interleave grain) and once as the FIFO ring with 512 KiB
+    chunks. GB/s figures are on the bytes the respective schedule moves."""
+    n, nbytes = 8, 64 << 20
+    res = {}
+    for label, env in (("direct", {"DFCCL_PROTO": "direct"}), ("fifo_512KiB_chunks", {"DFCCL_PROTO": "fifo"})):
+        r = run_native(["allreduce", "--ranks", n, "--bytes", nbytes, "--dtype", "bf16", "--iters", 10], env)
+        res[label] = {"ms": r["best_ms"], "median_ms": r["median_ms"], "algbw_GBps": r["algbw_GBps"],
+                      "busbw_GBps": r["busbw_GBps"], "moved_GBps": r["moved_GBps"],
+                      "frac_of_hbm_peak": round(r["moved_GBps"] / HBM_PEAK_GBPS, 4), "channels": r["channels"],
+                      "chunk_bytes": r["chunk_bytes"], "correct": r["correct"], "ctx_saves": r["ctx_saves"]}
+    res["workload"] = f"ring all-reduce, {n} virtual ranks x {nbytes >> 20} MiB bf16 Sum (time: submit on all ranks -> last callback)"
+    return res
+
+
+def bench_latency():
+    """SQE->CQE interval of 4 KiB fp16 all-reduces over 4 virtual ranks (taken inside the library: entry
+    written -> completion seen by the poller), all ranks submitting together."""
+    r = run_native(["latency", "--ranks", 4, "--bytes", 4096, "--dtype", "fp16", "--iters", 2000])
+    return {"workload": "4 virtual ranks, 4096 B fp16 Sum all-reduce, one host thread per rank",
+            "p50_us": r["p50_us"], "p90_us": r["p90_us"], "p99_us": r["p99_us"], "min_us": r["min_us"],
+            "correct": r["correct"]}
+
+
+def bench_disordered():
+    """256 registered fp16 all-reduces (4 KiB .. 4 MiB, log-uniform) over 4 virtual ranks, every rank submitting
+    in its own random order."""
+    r = run_native(["disorder", "--ranks", 4, "--colls", 256, "--dtype", "fp16"])
+    return {"workload": "256 all-reduces, 4 virtual ranks, sizes log-uniform 4 KiB..4 MiB fp16, per-rank random order",
+            "deadlocks": r["deadlocks"], "correct": r["correct"], "wall_ms": r["wall_ms"], "p50_us": r["p50_us"],
+            "p99_us": r["p99_us"], "preemptions": r["preemptions_ctx_saves"], "completions": r["cqes"]}
+
+
+def bench_buckets():
+    """40 gradient buckets of 25M elements over 4 virtual ranks, all submitted at once: bf16 Sum, then int32 Sum."""
+    out = {}
+    for dt in ("bf16", "int32"):
+        r = run_native(["buckets", "--ranks", 4, "--colls", 40, "--elems", 25000000, "--dtype", dt, "--iters", 3],
+                       timeout=300)
+        out[dt] = {"ms": r["best_ms"], "algbw_GBps": r["algbw_GBps"], "moved_GBps": r["moved_GBps"],
+                   "correct": r["correct"], "ctx_saves": r["ctx_saves"], "protocol": r["protocol"]}
+    return out
 
 
 def main():
@@ -194,6 +198,8 @@ def main():
     if not args.skip_daemon:
         line["daemon_all_reduce"] = bench_daemon_all_reduce()
         line["sqe_to_cqe_latency"] = bench_latency()
+        line["disordered_small_collectives"] = bench_disordered()
+        line["gradient_buckets"] = bench_buckets()
     if not args.skip_cpu:
         line["cpu_baseline"] = bench_cpu_baseline()
     print(json.dumps(line))

@@ -375,11 +375,15 @@ static int runBuckets(const Args& a, bool single) {
   w.destroy();
   const double best = ms.empty() ? 0 : *std::min_element(ms.begin(), ms.end());
   const double med = pct(ms, 0.5);
-  const double sched = (6.0 * n - 4.0) / n * (double)bytes * n * nc;  // bytes the FIFO ring schedule moves
+  // bytes the schedule moves, all ranks together: the FIFO ring reads and writes every staged slice
+  // ((6n-4)/n * N per rank), the direct protocol reads n chunks and writes one, then copies n-1 ((3n-1)/n * N)
+  const double perRank = geom.protocol == 1 ? (3.0 * n - 1.0) / n : (6.0 * n - 4.0) / n;
+  const double sched = perRank * (double)bytes * n * nc;
   printf("{\"mode\": \"%s\", \"ranks\": %d, \"colls\": %d, \"dtype\": \"%s\", \"bytes_per_rank_per_coll\": %zu, "
-         "\"channels\": %d, \"chunk_bytes\": %lld, \"iters\": %d, \"correct\": %s, \"best_ms\": %.4f, \"median_ms\": %.4f, "
-         "\"algbw_GBps\": %.1f, \"busbw_GBps\": %.1f, \"schedule_GBps\": %.1f, \"ctx_saves\": %llu}\n",
-         single ? "allreduce" : "buckets", n, nc, a.dtype.c_str(), bytes, geom.nChannels,
+         "\"protocol\": \"%s\", \"channels\": %d, \"chunk_bytes\": %lld, \"iters\": %d, \"correct\": %s, \"best_ms\": %.4f, "
+         "\"median_ms\": %.4f, \"algbw_GBps\": %.1f, \"busbw_GBps\": %.1f, \"moved_GBps\": %.1f, \"ctx_saves\": %llu}\n",
+         single ? "allreduce" : "buckets", n, nc, a.dtype.c_str(), bytes, geom.protocol == 1 ? "direct" : "fifo",
+         geom.nChannels,
          (long long)geom.chunkElems * es, a.iters, ok ? "true" : "false", best, med,
          best > 0 ? (double)bytes * nc / (best * 1e-3) / 1e9 : 0, best > 0 ? (double)bytes * nc / (best * 1e-3) / 1e9 * 2 * (n - 1) / n : 0,
          best > 0 ? sched / (best * 1e-3) / 1e9 : 0, (unsigned long long)st.ctxSaves);
