@@ -25,6 +25,9 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "oracle"))
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the headline kernel from the rocprofv3 --pmc runs recorded in
+# profiles/reduce_copy_f32_sum_k2_256MiB.md (FETCH_SIZE x 1.99974 + WRITE_SIZE x 1.00000, in KiB)
+TRAFFIC_BYTES_PER_LAUNCH = int(round((262164.1 * 1.99974 + 262144.0 * 1.00000) * 1024))
 
 
 def bench_reduce_copy(steps, warmup, nbytes=256 << 20, k=2):
@@ -191,7 +194,7 @@ def main():
                    "bytes_counted": "(k+1)*N*sizeof(T)", "correct": rc["correct"]},
         "frac_of_hbm_peak": round(gbps_wall / HBM_PEAK_GBPS, 4),
         "roofline": {"bound": "hbm", "achieved": round(gbps_kernel, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "reduceCopyKernel<f32,Sum,2>", "kernel_ms_avg": round(rc["kernel_ms_avg"], 5),
                      "kernel_ms_min": round(rc["kernel_ms_min"], 5)},
     }
