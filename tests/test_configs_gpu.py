@@ -1,0 +1,110 @@
+"""The benchmark configurations at full size, checked through size-independent properties: exact sums of small
+integers in every dtype (native driver, element-by-element verification on the host), zero deadlocks under
+per-rank random submission order, and bit-exact Max / Min under forced preemption with a concurrent GEMM stream."""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+import dfccl_oracle as orc
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DRIVER = os.path.join(ROOT, "dfccl_amd", "dfccl_bench")
+
+
+def native(args, env=None, timeout=240):
+    e = dict(os.environ, DFCCL_DAEMON_MAX_MS="20000")
+    e.update(env or {})
+    out = subprocess.run([DRIVER] + [str(a) for a in args], env=e, capture_output=True, text=True, timeout=timeout)
+    assert out.returncode == 0, out.stderr[-2000:]
+    return json.loads(out.stdout.strip().splitlines()[-1])
+
+
+@pytest.mark.parametrize("proto", ["direct", "fifo"])
+def test_config3_disordered_256_collectives_no_deadlock(proto):
+    # 256 registered fp16 all-reduces over 4 virtual ranks, sizes log-uniform 4 KiB..4 MiB, every rank submits in
+    # its own random permutation; every element of every result is verified (inputs are rank + 1, sum = 10)
+    r = native(["disorder", "--ranks", 4, "--colls", 256, "--dtype", "fp16", "--timeout", 60], {"DFCCL_PROTO": proto})
+    assert r["deadlocks"] == 0 and r["correct"] is True
+    assert r["cqes"] == 4 * 256
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "int32"])
+def test_config4_gradient_buckets_full_size(dtype):
+    # 4 virtual ranks, 40 buckets of 25,000,000 elements, all submitted at once; results verified element by element
+    r = native(["buckets", "--ranks", 4, "--colls", 40, "--elems", 25000000, "--dtype", dtype, "--iters", 1])
+    assert r["correct"] is True
+
+
+def test_config2_full_size_all_reduce_8_ranks_bf16():
+    for proto in ("direct", "fifo"):
+        r = native(["allreduce", "--ranks", 8, "--bytes", 64 << 20, "--dtype", "bf16", "--iters", 2],
+                   {"DFCCL_PROTO": proto})
+        assert r["correct"] is True and r["protocol"] == proto
+
+
+def test_latency_mode_small_collectives_correct():
+    r = native(["latency", "--ranks", 4, "--bytes", 4096, "--dtype", "fp16", "--iters", 200])
+    assert r["correct"] is True and r["p50_us"] > 0
+
+
+@pytest.mark.parametrize("proto", ["direct", "fifo"])
+def test_config5_preemption_under_gemm_contention(proto, monkeypatch):
+    # 8 virtual ranks, fp32 Max over 128 MiB and int8 Min over 128 MiB per rank, a bf16 8192^3 GEMM loop on another
+    # stream, forced quit / resume every 64 slices; results bit-exact against torch's own max / min and against
+    # the un-preempted run
+    from dfccl_amd.ring import VirtualRing
+    import dfccl_amd
+    n = 8
+    nf, ni = (128 << 20) // 4, 128 << 20
+    g = torch.Generator(device="cuda:0").manual_seed(5)
+    fsend = [torch.randn(nf, device="cuda:0", generator=g) for _ in range(n)]
+    isend = [torch.randint(-128, 128, (ni,), device="cuda:0", generator=g, dtype=torch.int8) for _ in range(n)]
+    fwant, iwant = fsend[0], isend[0]
+    for r in range(1, n):
+        fwant = torch.maximum(fwant, fsend[r])
+        iwant = torch.minimum(iwant, isend[r])
+    a = torch.randn(8192, 8192, device="cuda:0", dtype=torch.bfloat16)
+    b = torch.randn(8192, 8192, device="cuda:0", dtype=torch.bfloat16)
+    torch.cuda.synchronize()  # no daemon is resident yet
+    monkeypatch.setenv("DFCCL_PROTO", proto)
+    monkeypatch.setenv("DFCCL_DAEMON_MAX_MS", "20000")
+    results = {}
+    # a FIFO channel of this collective moves 15 steps x 2 slices of 256 KiB in all, fewer than 64: there the
+    # hook fires every 8 slices instead, so that every workgroup is preempted several times per collective
+    forced = "64" if proto == "direct" else "8"
+    for force in ("0", forced):
+        monkeypatch.setenv("DFCCL_FORCE_QUIT_EVERY", force)
+        frecv = [torch.zeros_like(t) for t in fsend]
+        irecv = [torch.zeros_like(t) for t in isend]
+        torch.cuda.current_stream().synchronize()
+        with VirtualRing(n) as ring:
+            ring.prepare(0, "all_reduce", nf, dfccl_amd.ncclFloat32, dfccl_amd.ncclMax)
+            ring.prepare(1, "all_reduce", ni, dfccl_amd.ncclInt8, dfccl_amd.ncclMin)
+            ring.finalize()
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                for _ in range(60):
+                    c = a @ b
+            for rep in range(2):
+                for r in range(n):
+                    ring.submit(r, 0, fsend[r], frecv[r])
+                    ring.submit(r, 1, isend[r], irecv[r])
+                ring.wait([(r, cid) for r in range(n) for cid in (0, 1)], timeout=90)
+            stats = ring.stats()
+            side.synchronize()
+        results[force] = (frecv, irecv, stats)
+        for r in range(n):
+            assert torch.equal(frecv[r], fwant), (force, r)
+            assert torch.equal(irecv[r], iwant), (force, r)
+        del c
+    assert results["0"][2]["forcedQuits"] == 0
+    s = results[forced][2]
+    assert s["forcedQuits"] > 0 and s["ctxSaves"] >= s["forcedQuits"]
+    for r in range(n):  # preempted run == un-preempted run, bit for bit
+        assert torch.equal(results["0"][0][r], results[forced][0][r])
+        assert torch.equal(results["0"][1][r], results[forced][1][r])

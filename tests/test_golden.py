@@ -1,0 +1,72 @@
+"""Golden vectors (tests/golden/ring_cases.npz, written by tests/golden/make_golden.py from the CPU oracle):
+the oracle must keep reproducing them (CPU), and the HIP path must match them (GPU).  The chunk geometry of
+each case is part of the fixture, so on the GPU only the cases whose geometry the library's planner also
+chooses for that size are compared bit for bit in float; integer and Min/Max cases do not depend on it."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "golden"))
+
+import dfccl_oracle as orc  # noqa: E402
+from make_golden import CASES, run_case  # noqa: E402
+
+DATA = np.load(os.path.join(HERE, "golden", "ring_cases.npz"), allow_pickle=False)
+
+
+def case_arrays(idx, n, kind):
+    sends = [DATA[f"c{idx}_in{r}"] for r in range(n)]
+    nout = 1 if kind == "reduce_copy" else n
+    outs = [DATA[f"c{idx}_out{r}"] for r in range(nout)]
+    return sends, outs
+
+
+@pytest.mark.parametrize("idx", range(len(CASES)))
+def test_oracle_reproduces_golden(idx):
+    kind, dtype, op, n, count, root, geom = CASES[idx]
+    sends, outs = case_arrays(idx, n, kind)
+    got = run_case(kind, dtype, op, n, count, root, geom, [s.copy() for s in sends])
+    for r in range(len(outs)):
+        assert np.array_equal(got[r], outs[r]), (idx, r)
+
+
+def order_independent(dtype, op):
+    return dtype in (orc.I8, orc.I32) or op in (orc.MAX, orc.MIN)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("idx", range(len(CASES)))
+def test_hip_path_matches_golden(idx, monkeypatch):
+    import torch
+    import dfccl_amd
+    from dfccl_amd.ring import VirtualRing
+    from gpu_util import TORCH_OF, to_gpu, to_np
+    kind, dtype, op, n, count, root, geom = CASES[idx]
+    sends_np, outs = case_arrays(idx, n, kind)
+    sends = [to_gpu(dtype, s) for s in sends_np]
+    if kind == "reduce_copy":
+        dst = torch.zeros(count, dtype=TORCH_OF[dtype], device="cuda:0")
+        dfccl_amd.reduce_copy(sends, dst, op)
+        torch.cuda.current_stream().synchronize()
+        assert np.array_equal(to_np(dtype, dst), outs[0])
+        return
+    monkeypatch.setenv("DFCCL_DAEMON_MAX_MS", "10000")
+    recv_len = count * n if kind == "all_gather" else count
+    recvs = [torch.zeros(recv_len, dtype=TORCH_OF[dtype], device="cuda:0") for _ in range(n)]
+    torch.cuda.current_stream().synchronize()
+    with VirtualRing(n) as ring:
+        ring.prepare(0, kind, count, dtype, op, root)
+        ring.finalize()
+        g = ring.ctxs[0].geometry(0)
+        same_geometry = (g.nChannels, g.chunkElems, g.alignElems) == geom
+        ring.run(0, sends, recvs, timeout=30)
+        copy_kind = kind in ("all_gather", "broadcast")
+        if not (copy_kind or order_independent(dtype, op) or same_geometry or kind in ("reduce_scatter", "reduce")):
+            pytest.skip("float all-reduce planned with another chunk geometry than the fixture's")
+        for r in range(n):
+            if kind == "reduce" and r != root:
+                continue
+            assert np.array_equal(to_np(dtype, recvs[r]), outs[r]), (idx, r)
