@@ -35,6 +35,8 @@ namespace dfccl {
 
 constexpr int kDaemonUnroll = 1;  // see reduce_copy.hip: shallow unrolling keeps DRAM accesses ordered
 constexpr int kReadyWords = (kMaxColls + 63) / 64;
+constexpr int kIdleDepth = 4;    // polls of the host ring an idle leader keeps in flight
+constexpr int kIdleRounds = 8;   // x kIdleDepth polls before the leader goes round its main loop again
 enum RunStatus : int { kRunDone = 0, kRunPreempted = 1 };
 
 // Geometry of the direct all-reduce sweeps: loop l covers elements [l * loop, (l + 1) * loop), split into
@@ -69,6 +71,7 @@ struct WgShared {
   int32_t waitOk;
   int32_t progressed;
   int32_t peersLoaded;
+  int32_t released;        // the results of this visit are already visible to the system
   int64_t threshold;
   int64_t slicesSinceLoad;
   CollPlan plan;
@@ -84,6 +87,30 @@ struct WgShared {
 
 #define DFCCL_AGENT __HIP_MEMORY_SCOPE_AGENT
 #define DFCCL_SYSTEM __HIP_MEMORY_SCOPE_SYSTEM
+
+// Everything the daemon touches outside LDS is global memory.  Pointers that were loaded from memory have the
+// generic address space as far as the compiler can tell, and accesses through them would be flat instructions
+// (slower, and they stop the compiler from keeping several loads in flight); these helpers say what they are.
+template <typename T>
+__device__ __forceinline__ DFCCL_GLOBAL T* G(T* p) {
+  return (DFCCL_GLOBAL T*)p;
+}
+template <typename T>
+__device__ __forceinline__ void loadStruct(T& dst, const T* src) {
+  static_assert(sizeof(T) % 8 == 0, "copied in 64-bit words");
+  const DFCCL_GLOBAL uint64_t* s = (const DFCCL_GLOBAL uint64_t*)src;
+  uint64_t* d = (uint64_t*)&dst;
+#pragma unroll
+  for (unsigned i = 0; i < sizeof(T) / 8; i++) d[i] = s[i];
+}
+template <typename T>
+__device__ __forceinline__ void storeStruct(T* dst, const T& src) {
+  static_assert(sizeof(T) % 8 == 0, "copied in 64-bit words");
+  DFCCL_GLOBAL uint64_t* d = (DFCCL_GLOBAL uint64_t*)dst;
+  const uint64_t* s = (const uint64_t*)&src;
+#pragma unroll
+  for (unsigned i = 0; i < sizeof(T) / 8; i++) d[i] = s[i];
+}
 
 __device__ __forceinline__ uint64_t waveMin64(uint64_t v) {
 #pragma unroll
@@ -115,14 +142,14 @@ __device__ __forceinline__ WaitDesc waitFor(const void* ptr, uint64_t value, int
 __device__ __forceinline__ void trace(const DaemonArgs& A, WgShared& sh, uint32_t ev, uint32_t arg) {
   if (A.trace == nullptr) return;
   const uint32_t i = sh.traceCount++;
-  uint64_t* rec = A.trace + ((size_t)sh.wgIndex * kTraceRecords + (i % kTraceRecords)) * 2;
+  DFCCL_GLOBAL uint64_t* rec = G(A.trace) + ((size_t)sh.wgIndex * kTraceRecords + (i % kTraceRecords)) * 2;
   rec[0] = (uint64_t)ev | ((uint64_t)arg << 32);
   rec[1] = wall_clock64();
 }
 
 // Writes the workgroup's counters to host-coherent memory (thread 0).
 __device__ __forceinline__ void flushStats(const RankDev& R, WgShared& sh, int ch) {
-  WgStats* out = &R.stats[ch];
+  DFCCL_GLOBAL WgStats* out = G(&R.stats[ch]);
   __hip_atomic_store(&out->sqesRead, sh.stats.sqesRead, __ATOMIC_RELAXED, DFCCL_SYSTEM);
   __hip_atomic_store(&out->cqesWritten, sh.stats.cqesWritten, __ATOMIC_RELAXED, DFCCL_SYSTEM);
   __hip_atomic_store(&out->ctxSaves, sh.stats.ctxSaves, __ATOMIC_RELAXED, DFCCL_SYSTEM);
@@ -154,10 +181,17 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
   const int pos = __builtin_popcountll(mm & ((1ull << lane) - 1ull));
   const int base = sh.numActive;
   if (mine && lane < take && base + pos < kMaxColls) {
-    DynCtx* d = &R.dyn[(size_t)ch * R.nColls + coll];
+    DFCCL_GLOBAL DynCtx* d = G(&R.dyn[(size_t)ch * R.nColls + coll]);
     d->sendbuff = sendbuff;
     d->recvbuff = recvbuff;
     d->active = 1;
+    if ((int32_t)coll == sh.loadedColl) {
+      // the collective whose context is resident starts its next instance: bring the resident copy up to date
+      sh.dyn.sendbuff = sendbuff;
+      sh.dyn.recvbuff = recvbuff;
+      sh.dyn.active = 1;
+      sh.peersLoaded = 0;
+    }
     sh.taskq[base + pos] = (uint16_t)coll;
   }
   if (lane == 0) {
@@ -170,8 +204,7 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
     sh.allFresh = (base == 0) ? 1 : 0;
     sh.stats.sqesRead += (uint64_t)consumed;
     sh.statsDirty = 1;
-    if (added > 0) sh.loadedColl = -1;  // a new instance may have changed the buffers of the cached context
-    if (R.nChannels > 1) __hip_atomic_store(&R.wgFrontier[ch], sh.frontier, __ATOMIC_RELAXED, DFCCL_AGENT);
+    if (R.nChannels > 1) __hip_atomic_store(G(&R.wgFrontier[ch]), sh.frontier, __ATOMIC_RELAXED, DFCCL_AGENT);
     trace(A, sh, kTrIngested, (uint32_t)consumed);
   }
 }
@@ -181,20 +214,56 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
 // from the registers, and pick up the host's control word.  (Role of sqRead, enqueue_ofccl_dev.cu:85-173.)
 __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, WgShared& sh, int lane) {
   const uint64_t base = sh.hostFrontier;
-  uint64_t w = 0;
-  bool valid = false;
-  if (lane < kSqesPerPoll * kSqeWords) {
-    const uint64_t ticket = base + (uint64_t)(lane >> 2);
-    const uint64_t* p = R.sq + ((ticket & (kSqRing - 1)) * kSqeWords + (lane & 3));
+  // With an empty task queue the leader has nothing to do but watch the ring's next entry and the control word
+  // (lanes 0..3 and lane 60, one load instruction).  It keeps kIdleDepth such polls in flight, so that a new
+  // entry is seen a fraction of a PCIe round trip after it lands rather than up to a whole one; the other
+  // entries of a burst are fetched by the next, ordinary poll.
+  const bool idleMode = sh.numActive == 0;
+  const int nlanes = idleMode ? kSqeWords : kSqesPerPoll * kSqeWords;
+  // every lane loads (the lanes without a word of their own re-read lane 0's, which costs nothing: it is the
+  // same request), so that no load is conditional and several can stay in flight
+  const uint64_t* pw = R.sq + ((base & (kSqRing - 1)) * kSqeWords);
+  if (lane < nlanes) pw = R.sq + (((base + (uint64_t)(lane >> 2)) & (kSqRing - 1)) * kSqeWords + (lane & 3));
+  else if (lane == 60) pw = (const uint64_t*)R.ctrl;  // the control word's allocation is 64 bytes long
+  const DFCCL_GLOBAL uint64_t* p = (const DFCCL_GLOBAL uint64_t*)pw;
+  const uint64_t tagWant = sqeTag(base + (uint64_t)(lane >> 2));
+  uint64_t w;
+  if (!idleMode) {
     w = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_SYSTEM);
-    valid = (w & ~kPtrMask) == sqeTag(ticket);
+  } else {
+    uint64_t q0 = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+    __builtin_amdgcn_s_sleep(4);
+    uint64_t q1 = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+    __builtin_amdgcn_s_sleep(4);
+    uint64_t q2 = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+    __builtin_amdgcn_s_sleep(4);
+    uint64_t q3 = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+    int polls = 0;
+    // one step: look at the oldest poll in flight; if it shows nothing, issue it again
+#define DFCCL_IDLE_STEP(q)                                                                                    \
+  {                                                                                                           \
+    w = q;                                                                                                    \
+    polls++;                                                                                                  \
+    const bool some = (lane < kSqeWords) ? ((w & ~kPtrMask) == tagWant) : (lane == 60 && (uint32_t)w != 0);   \
+    const uint64_t m = __ballot(some);                                                                        \
+    if ((m & 0xfull) == 0xfull || (m >> 60) != 0) break;                                                      \
+    __builtin_amdgcn_s_sleep(2);                                                                              \
+    q = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_SYSTEM);                                                 \
   }
-  uint32_t ctrl = 0;
-  if (lane == 60) ctrl = __hip_atomic_load(R.ctrl, __ATOMIC_RELAXED, DFCCL_SYSTEM);
-  ctrl = __shfl(ctrl, 60);
+    for (int it = 0; it < kIdleRounds; it++) {
+      DFCCL_IDLE_STEP(q0)
+      DFCCL_IDLE_STEP(q1)
+      DFCCL_IDLE_STEP(q2)
+      DFCCL_IDLE_STEP(q3)
+    }
+#undef DFCCL_IDLE_STEP
+    if (lane == 0 && polls > 1) sh.idle += polls - 1;
+  }
+  const bool valid = lane < nlanes && (w & ~kPtrMask) == tagWant;
+  const uint32_t ctrl = (uint32_t)__shfl(w, 60);
   if (ctrl != 0 && lane == 0) {
-    if (ctrl & kCtrlQuitRequest) __hip_atomic_store(&A.devFlags[0], 1u, __ATOMIC_RELAXED, DFCCL_AGENT);
-    if (ctrl & kCtrlAbort) __hip_atomic_store(&A.devFlags[1], 1u, __ATOMIC_RELAXED, DFCCL_AGENT);
+    if (ctrl & kCtrlQuitRequest) __hip_atomic_store(G(&A.devFlags[0]), 1u, __ATOMIC_RELAXED, DFCCL_AGENT);
+    if (ctrl & kCtrlAbort) __hip_atomic_store(G(&A.devFlags[1]), 1u, __ATOMIC_RELAXED, DFCCL_AGENT);
   }
   const uint64_t vm = __ballot(valid);
   int n = 0;
@@ -212,7 +281,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
     if (R.nChannels > 1) {
       if (lane < n) {
         const uint64_t ticket = base + (uint64_t)lane;
-        DevSqe* e = &R.mirror[ticket & (kSqRing - 1)];
+        DFCCL_GLOBAL DevSqe* e = G(&R.mirror[ticket & (kSqRing - 1)]);
         e->sendbuff = sendbuff;
         e->recvbuff = recvbuff;
         e->coll = coll;
@@ -221,7 +290,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
       }
       // every lane's entry is written before lane 0 publishes the new tail
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-      if (lane == 0) __hip_atomic_store(R.mirrorTail, base + (uint64_t)n, __ATOMIC_RELAXED, DFCCL_AGENT);
+      if (lane == 0) __hip_atomic_store(G(R.mirrorTail), base + (uint64_t)n, __ATOMIC_RELAXED, DFCCL_AGENT);
     }
     if (lane == 0) {
       sh.hostFrontier = base + (uint64_t)n;
@@ -235,11 +304,11 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
     uint64_t f = sh.frontier;
     if (R.nChannels > 1) {
       f = ~0ull;
-      if (lane < R.nChannels) f = __hip_atomic_load(&R.wgFrontier[lane], __ATOMIC_RELAXED, DFCCL_AGENT);
+      if (lane < R.nChannels) f = __hip_atomic_load(G(&R.wgFrontier[lane]), __ATOMIC_RELAXED, DFCCL_AGENT);
       f = waveMin64(f);
     }
     if (lane == 0 && f != sh.publishedHead) {
-      __hip_atomic_store(R.sqHead, f, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+      __hip_atomic_store(G(R.sqHead), f, __ATOMIC_RELAXED, DFCCL_SYSTEM);
       sh.publishedHead = f;
     }
   }
@@ -248,7 +317,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
 // Wave 0 of the other channels: take new entries from the mirror ring, one lane per entry.
 __device__ __forceinline__ void ingestMirror(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane) {
   const uint64_t f = sh.frontier;
-  const uint64_t tail = __hip_atomic_load(R.mirrorTail, __ATOMIC_ACQUIRE, DFCCL_AGENT);
+  const uint64_t tail = __hip_atomic_load(G(R.mirrorTail), __ATOMIC_ACQUIRE, DFCCL_AGENT);
   const int avail = (int)((tail - f) < 64 ? (tail - f) : 64);
   if (avail <= 0) {
     if (lane == 0) sh.ingested = 0;
@@ -258,15 +327,17 @@ __device__ __forceinline__ void ingestMirror(const DaemonArgs& A, const RankDev&
   e.sendbuff = e.recvbuff = 0;
   e.coll = 0;
   e.flags = 0;
-  if (lane < avail) e = R.mirror[(f + (uint64_t)lane) & (kSqRing - 1)];
+  if (lane < avail) loadStruct(e, &R.mirror[(f + (uint64_t)lane) & (kSqRing - 1)]);
   ingestEntries(A, R, sh, ch, lane, avail, e.sendbuff, e.recvbuff, e.coll, e.flags);
 }
 
 // One lane: is this parked collective's wait condition met?
 __device__ __forceinline__ bool descMet(const WaitDesc& w) {
-  for (int i = 0; i < w.count; i++) {
-    const uint64_t* p = (const uint64_t*)(uintptr_t)(w.ptr + (uint64_t)((int64_t)i * w.stride));
-    if (__hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_AGENT) < w.value) return false;
+  const bool tagged = (w.count & kWaitTagged) != 0;
+  const int count = w.count & (kWaitTagged - 1);
+  for (int i = 0; i < count; i++) {
+    const DFCCL_GLOBAL uint64_t* p = (const DFCCL_GLOBAL uint64_t*)(uintptr_t)(w.ptr + (uint64_t)((int64_t)i * w.stride));
+    if (!waitReached(__hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_AGENT), w.value, tagged)) return false;
   }
   return true;
 }
@@ -288,8 +359,10 @@ __device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, int ch
     const int i = base + lane;
     bool ready = false;
     if (i < n) {
+      WaitDesc w0, w1;
       const DynCtx* d = &R.dyn[(size_t)ch * R.nColls + sh.taskq[i]];
-      const WaitDesc w0 = d->wait[0], w1 = d->wait[1];
+      loadStruct(w0, &d->wait[0]);
+      loadStruct(w1, &d->wait[1]);
       ready = descMet(w0) && descMet(w1);
     }
     const uint64_t m = __ballot(ready);
@@ -302,12 +375,13 @@ __device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, int ch
 // Wave 0: wait until both conditions hold.  Lanes 0..31 watch the counters of
 // w0, lanes 32..63 those of w1; the ballot decides for the whole wave.  The wait
 // is bounded: when the budget is spent the collective is preempted.  (Role of
-// waitPeer, src/collectives_ofccl/device/ofccl_prims_simple.h:90-198.)
-__device__ __forceinline__ void waitDescs(const DaemonArgs& A, WgShared& sh, int lane, const WaitDesc& w0,
-                                          const WaitDesc& w1, bool adapt) {
+// waitPeer, src/collectives_ofccl/device/ofccl_prims_simple.h:90-198.)  Returns the word the lane saw last.
+__device__ __forceinline__ uint64_t waitDescs(const DaemonArgs& A, WgShared& sh, int lane, const WaitDesc& w0,
+                                              const WaitDesc& w1, bool adapt) {
   bool ok;
   int64_t spins = 0;
-  if (lane == 0) trace(A, sh, kTrWaitBegin, (uint32_t)(w0.count + w1.count));
+  uint64_t seen = 0;
+  if (lane == 0) trace(A, sh, kTrWaitBegin, (uint32_t)((w0.count + w1.count) & 0xffff));
   const int64_t forceEvery = A.knobs.forceQuitEvery;
   if (forceEvery > 0 && sh.slicesSinceLoad >= forceEvery) {
     ok = false;
@@ -315,13 +389,18 @@ __device__ __forceinline__ void waitDescs(const DaemonArgs& A, WgShared& sh, int
   } else {
     const WaitDesc& w = (lane < 32) ? w0 : w1;
     const int idx = lane & 31;
-    const uint64_t* p = nullptr;
-    if (idx < w.count) p = (const uint64_t*)(uintptr_t)(w.ptr + (uint64_t)((int64_t)idx * w.stride));
+    const bool tagged = (w.count & kWaitTagged) != 0;
+    const DFCCL_GLOBAL uint64_t* p = nullptr;
+    if (idx < (w.count & (kWaitTagged - 1)))
+      p = (const DFCCL_GLOBAL uint64_t*)(uintptr_t)(w.ptr + (uint64_t)((int64_t)idx * w.stride));
     const uint64_t need = w.value;
     bool ready = (p == nullptr);
     const int64_t threshold = sh.threshold;
     for (;;) {
-      if (!ready) ready = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_AGENT) >= need;
+      if (!ready) {
+        seen = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_AGENT);
+        ready = waitReached(seen, need, tagged);
+      }
       if (__ballot(!ready) == 0) { ok = true; break; }
       if (++spins >= threshold) { ok = false; break; }
       __builtin_amdgcn_s_sleep(1);
@@ -341,6 +420,7 @@ __device__ __forceinline__ void waitDescs(const DaemonArgs& A, WgShared& sh, int
       sh.dyn.wait[1] = w1;
     }
   }
+  return seen;
 }
 
 // ---------------------------------------------------------------- data movement
@@ -658,8 +738,8 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
           __syncthreads();  // every thread's loads and stores of this slice are done
           if (tid == 0) {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            if (d.send) __hip_atomic_store(&P.sendFlags[ch].tail, sendStep + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
-            if (d.recv) __hip_atomic_store(&P.recvFlags[ch].head, recvStep + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
+            if (d.send) __hip_atomic_store(G(&P.sendFlags[ch].tail), sendStep + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
+            if (d.recv) __hip_atomic_store(G(&P.recvFlags[ch].head), recvStep + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
             trace(A, sh, kTrPosted, (uint32_t)s);
             sh.progressed = 1;
             sh.slicesSinceLoad++;
@@ -716,21 +796,23 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
   int phase = sh.dyn.step;
   __syncthreads();  // every thread has taken its copy of the position before thread 0 changes it
 
-  if (!published && tid == 0) {
-    myPub->sendbuff = sendbuff;
-    myPub->recvbuff = recvbuff;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    __hip_atomic_store(&myPub->seq, inst + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
-    sh.dyn.slice = 1;
+  if (!published && tid < 2) {
+    // the words carry their own instance tag: no ordering between them is needed, and the buffers' contents
+    // were made visible by whoever wrote them before the submission
+    const uint64_t tag = pubTag(inst);
+    __hip_atomic_store(G(tid == 0 ? &myPub->send : &myPub->recv), (tid == 0 ? sendbuff : recvbuff) | tag,
+                       __ATOMIC_RELAXED, DFCCL_AGENT);
+    if (tid == 0) sh.dyn.slice = 1;
   }
   if (!peersLoaded) {
-    const WaitDesc w0 = waitFor(&P.pubs[ch].seq, inst + 1, pubStride, n);
+    // lanes 0..n-1 watch the peers' send words, lanes 32..32+n-1 their receive words
+    const WaitDesc w0 = waitFor(&P.pubs[ch].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
+    const WaitDesc w1 = waitFor(&P.pubs[ch].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
     if (wave == 0) {
-      waitDescs(A, sh, lane, w0, noWait(), true);
-      if (sh.waitOk && lane < n) {
-        const PeerPub* pp = &P.pubs[(size_t)lane * C + ch];
-        sh.peerSend[lane] = pp->sendbuff;
-        sh.peerRecv[lane] = pp->recvbuff;
+      const uint64_t word = waitDescs(A, sh, lane, w0, w1, true);
+      if (sh.waitOk && (lane & 31) < n) {
+        if (lane < 32) sh.peerSend[lane] = word & kPtrMask;
+        else sh.peerRecv[lane & 31] = word & kPtrMask;
       }
       if (sh.waitOk && lane == 0) sh.peersLoaded = 1;
     }
@@ -749,8 +831,10 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
       __syncthreads();
       if (tid == 0) {
         trace(A, sh, kTrMoveEnd, 0);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        __hip_atomic_store(&P.p2[(size_t)me * C + ch], base + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
+        // released to the system here, while the peers are still busy, so that the completion need not wait for it
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+        if (!inPlace) sh.released = 1;
+        __hip_atomic_store(G(&P.p2[(size_t)me * C + ch]), base + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
         trace(A, sh, kTrPosted, 2);
         sh.progressed = 1;
         sh.slicesSinceLoad++;
@@ -835,7 +919,7 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
     if (tid == 0) {
       trace(A, sh, kTrMoveEnd, 0);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-      __hip_atomic_store(&P.p1[(size_t)me * C + ch], base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
+      __hip_atomic_store(G(&P.p1[(size_t)me * C + ch]), base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
       trace(A, sh, kTrPosted, 1);
       for (int t = 0; t < kMaxDirectRanks; t++) sh.sweep.peer[t] = (t < n) ? sh.peerRecv[t] : 0;
     }
@@ -888,8 +972,9 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
     __syncthreads();
     if (tid == 0) {
       trace(A, sh, kTrMoveEnd, 1);
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-      __hip_atomic_store(&P.p2[(size_t)me * C + ch], base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+      sh.released = 1;
+      __hip_atomic_store(G(&P.p2[(size_t)me * C + ch]), base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
       trace(A, sh, kTrPosted, 2);
     }
   }
@@ -927,8 +1012,8 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
   DynCtx* dynG = &R.dyn[(size_t)ch * R.nColls + coll];
   if (tid == 0) {
     if (sh.loadedColl != (int32_t)coll) {
-      sh.plan = R.plans[coll];
-      sh.dyn = *dynG;
+      loadStruct(sh.plan, &R.plans[coll]);
+      loadStruct(sh.dyn, dynG);
       sh.loadedColl = (int32_t)coll;
       sh.peersLoaded = 0;
       sh.stats.ctxLoads++;
@@ -941,6 +1026,7 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
     sh.threshold = thr < 1 ? 1 : thr;
     sh.waitOk = 1;
     sh.progressed = 0;
+    sh.released = 0;
     sh.slicesSinceLoad = 0;
     sh.dyn.wait[0] = noWait();
     sh.dyn.wait[1] = noWait();
@@ -962,28 +1048,29 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
       sh.dyn.wait[0] = noWait();
       sh.dyn.wait[1] = noWait();
       sh.taskq[qi] = (uint16_t)kInvalidTask;
+      sh.peersLoaded = 0;
       // completion (manipulateCQ7ResetDoneColl, enqueue_ofccl_dev.cu:773-920): results are released to the
-      // system, then the last channel to finish posts the entry
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+      // system (unless the protocol has done so already), then the last channel to finish posts the entry
+      if (!sh.released) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
       bool last = true;
       if (sh.plan.nChannels > 1) {
-        const uint64_t old = __hip_atomic_fetch_add(sh.plan.doneCounter, 1ull, __ATOMIC_ACQ_REL, DFCCL_AGENT);
+        const uint64_t old = __hip_atomic_fetch_add(G(sh.plan.doneCounter), 1ull, __ATOMIC_ACQ_REL, DFCCL_AGENT);
         last = ((old + 1) % (uint64_t)sh.plan.nChannels == 0);
       }
       if (last) {
         // a rank with a single channel has a single poster, which keeps the ticket itself
         const uint64_t t = (R.nChannels == 1) ? sh.cqNext++
-                                              : __hip_atomic_fetch_add(R.cqTicket, 1ull, __ATOMIC_RELAXED, DFCCL_AGENT);
-        __hip_atomic_store(&R.cq[t & (kCqRing - 1)],
+                                              : __hip_atomic_fetch_add(G(R.cqTicket), 1ull, __ATOMIC_RELAXED, DFCCL_AGENT);
+        __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]),
                            cqeEncode((unsigned)ch, (unsigned)(t + 1), (unsigned)sh.plan.collId), __ATOMIC_RELEASE,
                            DFCCL_SYSTEM);
         sh.stats.cqesWritten++;
         trace(A, sh, kTrCqePosted, coll);
       }
-      *dynG = sh.dyn;
+      storeStruct(dynG, sh.dyn);
     } else {
       // preempted: save the context (saveExcutingCollCtx, enqueue_ofccl_dev.cu:664-677)
-      *dynG = sh.dyn;
+      storeStruct(dynG, sh.dyn);
       sh.stats.ctxSaves++;
     }
     trace(A, sh, kTrVisitEnd, (uint32_t)status);
@@ -1004,7 +1091,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
   const uint64_t startTick = wall_clock64();
 
   // ---- restore the state a previous launch saved (blockInit, enqueue_ofccl_dev.cu:203-479)
-  WgSaved& S = R.saved[ch];
+  DFCCL_GLOBAL WgSaved& S = *G(&R.saved[ch]);
   if (tid == 0) {
     sh.frontier = S.frontier;
     sh.hostFrontier = S.hostFrontier;
@@ -1024,7 +1111,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     sh.allFresh = 0;
     sh.cqNext = S.cqNext;
     trace(A, sh, kTrLaunch, A.epoch);
-    const WgStats* hs = &R.stats[ch];
+    const DFCCL_GLOBAL WgStats* hs = G(&R.stats[ch]);
     sh.stats.sqesRead = hs->sqesRead;
     sh.stats.cqesWritten = hs->cqesWritten;
     sh.stats.ctxSaves = hs->ctxSaves;
@@ -1037,7 +1124,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
   }
   __syncthreads();
   for (int i = tid; i < sh.numActive; i += kWgThreads) sh.taskq[i] = S.taskq[i];
-  for (int i = tid; i < R.nColls; i += kWgThreads) sh.collChannels[i] = (uint8_t)R.plans[i].nChannels;
+  for (int i = tid; i < R.nColls; i += kWgThreads) sh.collChannels[i] = (uint8_t)G(&R.plans[i])->nChannels;
   __syncthreads();
 
   for (;;) {
@@ -1052,8 +1139,8 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
         uint32_t abortFlag = 0, quitFlag = 0;
         bool expired = false;
         if ((sh.round++ & 7u) == 0) {
-          abortFlag = __hip_atomic_load(&A.devFlags[1], __ATOMIC_RELAXED, DFCCL_AGENT);
-          quitFlag = __hip_atomic_load(&A.devFlags[0], __ATOMIC_RELAXED, DFCCL_AGENT);
+          abortFlag = __hip_atomic_load(G(&A.devFlags[1]), __ATOMIC_RELAXED, DFCCL_AGENT);
+          quitFlag = __hip_atomic_load(G(&A.devFlags[0]), __ATOMIC_RELAXED, DFCCL_AGENT);
           expired = K.maxLifetimeTicks > 0 && (int64_t)(wall_clock64() - startTick) > K.maxLifetimeTicks;
         }
         if (sh.ingested > 0 || sh.progressedRound) sh.idle = 0;
@@ -1121,10 +1208,10 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
   if (tid == 0) {
     trace(A, sh, kTrExit, (uint32_t)exitKind);
     if (A.trace != nullptr)  // the last record slot of the workgroup holds how many records it wrote
-      A.trace[((size_t)sh.wgIndex * kTraceRecords + (kTraceRecords - 1)) * 2 + 1] = sh.traceCount;
+      G(A.trace)[((size_t)sh.wgIndex * kTraceRecords + (kTraceRecords - 1)) * 2 + 1] = sh.traceCount;
     flushStats(R, sh, ch);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-    __hip_atomic_store(&R.wgExit[ch], (A.epoch << 4) | (uint32_t)exitKind, __ATOMIC_RELEASE, DFCCL_SYSTEM);
+    __hip_atomic_store(G(&R.wgExit[ch]), (A.epoch << 4) | (uint32_t)exitKind, __ATOMIC_RELEASE, DFCCL_SYSTEM);
   }
 }
 

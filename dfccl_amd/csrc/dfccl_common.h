@@ -68,23 +68,31 @@ struct alignas(128) ConnFlags {
 // Direct protocol: what a rank's workgroup publishes when it starts an instance
 // of a collective, so that its peers can read its buffers in place (the role of
 // the reference's ptrExchange, src/collectives_ofccl/device/ofccl_prims_simple.h:737-869).
+// Each word carries the instance it belongs to in its top 16 bits (pubTag), so a peer that polls the word
+// gets the pointer with the same load that tells it the instance has started.
 struct alignas(32) PeerPub {
-  uint64_t seq;        // instances started, written last
-  uint64_t sendbuff;
-  uint64_t recvbuff;
-  uint64_t pad;
+  uint64_t send;       // sendbuff | pubTag(instance)
+  uint64_t recv;       // recvbuff | pubTag(instance)
+  uint64_t pad[2];
 };
+DFCCL_HD uint64_t pubTag(uint64_t instance) { return ((instance + 1) & 0xffffull) << 48; }
 
 // A wait condition: all of `count` 64-bit counters at ptr, ptr + stride, ... have
 // reached `value`.  Every blocking point of both protocols is expressed as (at
 // most) two of these, which lets the scheduler test the readiness of a parked
 // collective without loading its context.
+// With kWaitTagged set in `count` the words are tagged pointers instead: the condition is that the top 16
+// bits of every word have reached `value` in modular (16-bit window) order.
 struct WaitDesc {
   uint64_t ptr;
   uint64_t value;
   int32_t stride;  // bytes
-  int32_t count;   // 0 = no condition
+  int32_t count;   // 0 = no condition; may carry kWaitTagged
 };
+constexpr int32_t kWaitTagged = 0x10000;
+DFCCL_HD bool waitReached(uint64_t word, uint64_t value, bool tagged) {
+  return tagged ? (int16_t)((uint16_t)(word >> 48) - (uint16_t)value) >= 0 : word >= value;
+}
 
 enum Proto : int { kProtoFifo = 0, kProtoDirect = 1 };
 constexpr int kMaxDirectRanks = 8;           // ranks whose buffers one workgroup folds in a single pass

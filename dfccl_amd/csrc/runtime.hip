@@ -147,6 +147,7 @@ struct ofcclRankCtx {
   std::atomic<uint64_t> submitted{0}, completed{0};
   std::thread poller;
   std::atomic<bool> stopPoller{false};
+  std::atomic<bool> pollerAsleep{false};
   std::mutex pollMu;
   std::condition_variable pollCv;
 };
@@ -532,11 +533,14 @@ static void pollerLoop(ofcclRankCtx* c) {
       continue;
     }
     if (c->submitted.load(std::memory_order_acquire) == c->completed.load(std::memory_order_acquire)) {
+      // nothing outstanding: sleep at once. (Spinning on here was measured: it gains nothing for a caller that
+      // submits again right away, and with as many rank contexts as cores it starves the submitting threads.)
       std::unique_lock<std::mutex> lk(c->pollMu);
+      c->pollerAsleep.store(true);  // sequentially consistent, as is the submitter's increment: one sees the other
       c->pollCv.wait_for(lk, std::chrono::milliseconds(2), [&] {
-        return c->stopPoller.load(std::memory_order_acquire) ||
-               c->submitted.load(std::memory_order_acquire) != c->completed.load(std::memory_order_acquire);
+        return c->stopPoller.load() || c->submitted.load() != c->completed.load();
       });
+      c->pollerAsleep.store(false);
       emptySpins = 0;
     } else if (++emptySpins > 20000) {
       sched_yield();
@@ -579,7 +583,7 @@ static ncclResult_t runColl(const void* sendbuff, void* recvbuff, int collId, Ca
   }
   c->callbacks[collId] = cb;
   c->cbArgs[collId] = cbArgs;
-  c->submitted.fetch_add(1, std::memory_order_acq_rel);
+  c->submitted.fetch_add(1);
   while (sqWrite(c, (uint64_t)(uintptr_t)sendbuff, (uint64_t)(uintptr_t)recvbuff, (uint32_t)c->collIndex[collId], 0) ==
          -1) {
     sched_yield();
@@ -596,7 +600,11 @@ static ncclResult_t runColl(const void* sendbuff, void* recvbuff, int collId, Ca
       d->cv.notify_all();
     }
   }
-  c->pollCv.notify_one();
+  if (c->pollerAsleep.load()) {
+    // taking the mutex orders this notification after the poller's test of the predicate
+    { std::lock_guard<std::mutex> lk(c->pollMu); }
+    c->pollCv.notify_one();
+  }
   return ncclSuccess;
 }
 
