@@ -26,7 +26,7 @@ class Stats(ctypes.Structure):
 class CollGeometry(ctypes.Structure):
     _fields_ = [("nRanks", ctypes.c_int), ("nChannels", ctypes.c_int), ("chunkElems", ctypes.c_int64),
                 ("alignElems", ctypes.c_int64), ("sliceElems", ctypes.c_int64), ("slicesPerChunk", ctypes.c_int),
-                ("fifoSlots", ctypes.c_int), ("protocol", ctypes.c_int), ("oneShot", ctypes.c_int)]
+                ("fifoSlots", ctypes.c_int), ("protocol", ctypes.c_int)]
 
 
 # every symbol include/ofccl.h declares: name -> (restype, argtypes)

@@ -347,6 +347,7 @@ static int runBuckets(const Args& a, bool single) {
   std::vector<uint64_t> tStart(total), tStop(total);
   std::vector<std::atomic<uint64_t>> endNs(total);
   for (auto& e : endNs) e.store(0);
+  std::vector<double> lastSubmit(n, 0), lastComplete(n, 0), lastSeen(n, 0);
   std::vector<std::thread> th;
   for (int r = 0; r < n; r++) {
     th.emplace_back([&, r] {
@@ -361,6 +362,13 @@ static int runBuckets(const Args& a, bool single) {
           if (!waitFlag(flags[(size_t)r * nc + c], a.timeoutS)) { failed.store(1); fprintf(stderr, "rank %d coll %d timed out\n", r, c); return; }
         uint64_t t = nowNs(), prev = endNs[it].load();
         while (prev < t && !endNs[it].compare_exchange_weak(prev, t)) {}
+        if (it == total - 1) {
+          uint64_t sN = 0, cN = 0;
+          NK(dfcclGetCollTiming(w.ctx[r], nc - 1, &sN, &cN));
+          lastSubmit[r] = (double)(sN - tStart[it]) / 1000.0;
+          lastComplete[r] = (double)(cN - tStart[it]) / 1000.0;
+          lastSeen[r] = (double)(t - tStart[it]) / 1000.0;
+        }
         bar.wait();
       }
     });
@@ -375,9 +383,16 @@ static int runBuckets(const Args& a, bool single) {
   w.destroy();
   const double best = ms.empty() ? 0 : *std::min_element(ms.begin(), ms.end());
   const double med = pct(ms, 0.5);
+  if (getenv("DFCCL_BENCH_VERBOSE")) {
+    // last iteration, microseconds after rank 0's start stamp: last entry written, last completion seen by the
+    // poller, waiting thread released
+    for (int r = 0; r < n; r++)
+      fprintf(stderr, "rank %d: submitted %.1f  completion seen %.1f  thread released %.1f (iteration %.1f)\n", r,
+              lastSubmit[r], lastComplete[r], lastSeen[r], ms.empty() ? 0.0 : ms.back() * 1000.0);
+  }
   // bytes the schedule moves, all ranks together: the FIFO ring reads and writes every staged slice
-  // ((6n-4)/n * N per rank), the direct protocol reads n chunks and writes one, then copies n-1 ((3n-1)/n * N)
-  const double perRank = geom.protocol == 1 ? (3.0 * n - 1.0) / n : (6.0 * n - 4.0) / n;
+  // ((6n-4)/n * N per rank), the direct protocol reads every input once and writes every output once (2 N)
+  const double perRank = geom.protocol == 1 ? 2.0 : (6.0 * n - 4.0) / n;
   const double sched = perRank * (double)bytes * n * nc;
   printf("{\"mode\": \"%s\", \"ranks\": %d, \"colls\": %d, \"dtype\": \"%s\", \"bytes_per_rank_per_coll\": %zu, "
          "\"protocol\": \"%s\", \"channels\": %d, \"chunk_bytes\": %lld, \"iters\": %d, \"correct\": %s, \"best_ms\": %.4f, "

@@ -35,8 +35,6 @@ namespace dfccl {
 
 constexpr int kDaemonUnroll = 1;  // see reduce_copy.hip: shallow unrolling keeps DRAM accesses ordered
 constexpr int kReadyWords = (kMaxColls + 63) / 64;
-constexpr int kIdleDepth = 4;    // polls of the host ring an idle leader keeps in flight
-constexpr int kIdleRounds = 8;   // x kIdleDepth polls before the leader goes round its main loop again
 enum RunStatus : int { kRunDone = 0, kRunPreempted = 1 };
 
 // Geometry of the direct all-reduce sweeps: loop l covers elements [l * loop, (l + 1) * loop), split into
@@ -45,8 +43,8 @@ struct SweepGeom {
   int64_t count, loop, chunkElems, alignElems;
   int n, C, ch, es;
   int me, dtype, op, pad;
-  uint64_t dst;                      // my receive buffer
-  uint64_t peer[kMaxDirectRanks];    // phase 0: the send buffers in fold order; phase 1: the receive buffers by rank
+  uint64_t src[kMaxDirectRanks];     // the send buffers in fold order: in[me + 1], in[me + 2], ..., in[me]
+  uint64_t dst[kMaxDirectRanks];     // every rank's receive buffer
 };
 struct WgShared {
   // scheduler state
@@ -61,10 +59,12 @@ struct WgShared {
   int32_t ingested;
   int32_t progressedRound;
   int32_t loadedColl;      // collective whose plan and position are in LDS, -1: none
-  int32_t statsDirty;
+  uint32_t statsEpoch;     // last request for the counters this workgroup has answered
+  uint32_t statsReqSeen;   // leader: last request number passed on to the other workgroups
   uint32_t traceCount;
   uint32_t wgIndex;
   uint32_t round;          // scheduler rounds since launch
+  int32_t rankBusy;        // leader: other channels of the rank still have work in flight
   int32_t allFresh;        // every collective of the task queue was ingested this round (nothing is parked)
   uint64_t cqNext;         // single-channel ranks: next completion ticket
   // collective being run
@@ -77,8 +77,6 @@ struct WgShared {
   CollPlan plan;
   DynCtx dyn;
   WgStats stats;
-  uint64_t peerSend[kMaxDirectRanks];
-  uint64_t peerRecv[kMaxDirectRanks];
   SweepGeom sweep;         // arguments of the direct protocol's sweeps
   uint64_t ready[kReadyWords];
   uint16_t taskq[kMaxColls];
@@ -147,8 +145,8 @@ __device__ __forceinline__ void trace(const DaemonArgs& A, WgShared& sh, uint32_
   rec[1] = wall_clock64();
 }
 
-// Writes the workgroup's counters to host-coherent memory (thread 0).
-__device__ __forceinline__ void flushStats(const RankDev& R, WgShared& sh, int ch) {
+// Writes the workgroup's counters to host-coherent memory (thread 0), marked as the answer to request `epoch`.
+__device__ __forceinline__ void flushStats(const RankDev& R, WgShared& sh, int ch, uint32_t epoch) {
   DFCCL_GLOBAL WgStats* out = G(&R.stats[ch]);
   __hip_atomic_store(&out->sqesRead, sh.stats.sqesRead, __ATOMIC_RELAXED, DFCCL_SYSTEM);
   __hip_atomic_store(&out->cqesWritten, sh.stats.cqesWritten, __ATOMIC_RELAXED, DFCCL_SYSTEM);
@@ -158,7 +156,7 @@ __device__ __forceinline__ void flushStats(const RankDev& R, WgShared& sh, int c
   __hip_atomic_store(&out->forcedQuits, sh.stats.forcedQuits, __ATOMIC_RELAXED, DFCCL_SYSTEM);
   __hip_atomic_store(&out->slicesMoved, sh.stats.slicesMoved, __ATOMIC_RELAXED, DFCCL_SYSTEM);
   __hip_atomic_store(&out->spins, sh.stats.spins, __ATOMIC_RELAXED, DFCCL_SYSTEM);
-  sh.statsDirty = 0;
+  __hip_atomic_store(&out->epoch, (uint64_t)epoch, __ATOMIC_RELEASE, DFCCL_SYSTEM);
 }
 
 // Wave 0: append the entries held one per lane (lanes < avail) to the task queue if this channel takes part
@@ -203,7 +201,6 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
     sh.ingested = consumed;
     sh.allFresh = (base == 0) ? 1 : 0;
     sh.stats.sqesRead += (uint64_t)consumed;
-    sh.statsDirty = 1;
     if (R.nChannels > 1) __hip_atomic_store(G(&R.wgFrontier[ch]), sh.frontier, __ATOMIC_RELAXED, DFCCL_AGENT);
     trace(A, sh, kTrIngested, (uint32_t)consumed);
   }
@@ -215,10 +212,18 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
 __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, WgShared& sh, int lane) {
   const uint64_t base = sh.hostFrontier;
   // With an empty task queue the leader has nothing to do but watch the ring's next entry and the control word
-  // (lanes 0..3 and lane 60, one load instruction).  It keeps kIdleDepth such polls in flight, so that a new
+  // (lanes 0..3 and lane 60, one load instruction).  It keeps four such polls in flight, so that a new
   // entry is seen a fraction of a PCIe round trip after it lands rather than up to a whole one; the other
   // entries of a burst are fetched by the next, ordinary poll.
-  const bool idleMode = sh.numActive == 0;
+  // Not while other channels of the rank are still moving data, though: reads of host memory that are in
+  // flight hold up the memory requests of every workgroup on the same XCD.  The rank is busy while it has
+  // posted fewer completions than it has fetched submissions; then the leader polls once, and rarely.
+  const int idleRounds = (int)A.knobs.idlePollRounds;
+  bool busy = false;
+  if (sh.numActive == 0 && R.nChannels > 1)
+    busy = __hip_atomic_load(G(R.cqTicket), __ATOMIC_RELAXED, DFCCL_AGENT) < base;
+  if (lane == 0) sh.rankBusy = busy ? 1 : 0;
+  const bool idleMode = sh.numActive == 0 && idleRounds > 0 && !busy;
   const int nlanes = idleMode ? kSqeWords : kSqesPerPoll * kSqeWords;
   // every lane loads (the lanes without a word of their own re-read lane 0's, which costs nothing: it is the
   // same request), so that no load is conditional and several can stay in flight
@@ -250,7 +255,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
     __builtin_amdgcn_s_sleep(2);                                                                              \
     q = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_SYSTEM);                                                 \
   }
-    for (int it = 0; it < kIdleRounds; it++) {
+    for (int it = 0; it < idleRounds; it++) {
       DFCCL_IDLE_STEP(q0)
       DFCCL_IDLE_STEP(q1)
       DFCCL_IDLE_STEP(q2)
@@ -260,7 +265,12 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
     if (lane == 0 && polls > 1) sh.idle += polls - 1;
   }
   const bool valid = lane < nlanes && (w & ~kPtrMask) == tagWant;
-  const uint32_t ctrl = (uint32_t)__shfl(w, 60);
+  const uint64_t ctrlWord = __shfl(w, 60);
+  const uint32_t ctrl = (uint32_t)ctrlWord, statsReq = (uint32_t)(ctrlWord >> 32);
+  if (lane == 0 && statsReq != sh.statsReqSeen) {
+    sh.statsReqSeen = statsReq;
+    __hip_atomic_store(G(&A.devFlags[2]), statsReq, __ATOMIC_RELAXED, DFCCL_AGENT);
+  }
   if (ctrl != 0 && lane == 0) {
     if (ctrl & kCtrlQuitRequest) __hip_atomic_store(G(&A.devFlags[0]), 1u, __ATOMIC_RELAXED, DFCCL_AGENT);
     if (ctrl & kCtrlAbort) __hip_atomic_store(G(&A.devFlags[1]), 1u, __ATOMIC_RELAXED, DFCCL_AGENT);
@@ -317,12 +327,14 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
 // Wave 0 of the other channels: take new entries from the mirror ring, one lane per entry.
 __device__ __forceinline__ void ingestMirror(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane) {
   const uint64_t f = sh.frontier;
-  const uint64_t tail = __hip_atomic_load(G(R.mirrorTail), __ATOMIC_ACQUIRE, DFCCL_AGENT);
+  // polled with a relaxed load: an acquire would invalidate the L2 on every poll of every idle workgroup
+  const uint64_t tail = __hip_atomic_load(G(R.mirrorTail), __ATOMIC_RELAXED, DFCCL_AGENT);
   const int avail = (int)((tail - f) < 64 ? (tail - f) : 64);
   if (avail <= 0) {
     if (lane == 0) sh.ingested = 0;
     return;
   }
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   DevSqe e;
   e.sendbuff = e.recvbuff = 0;
   e.coll = 0;
@@ -483,17 +495,19 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
   return (uint64_t)lo | ((uint64_t)hi << 32);
 }
 
-// dst[off..] = src[0][off..] (op) src[1][off..] ... (op) src[n-1][off..], folded left to right with every
-// step rounded to the storage type: with src = in[c+1], in[c+2], ..., in[c] this is the ring's order for a
-// chunk owned by rank c.  n <= NS <= kMaxDirectRanks; the NS - n surplus loads re-read src[0] (they hit in
-// cache) so that every array element is defined: predicated loads made the compiler keep the packs in scratch.
+// dst[k][off..] = src[0][off..] (op) src[1][off..] ... (op) src[n-1][off..] for every k < n, folded left to
+// right with every step rounded to the storage type: with src = in[c+1], in[c+2], ..., in[c] this is the ring's
+// order for a chunk owned by rank c.  n <= NS <= kMaxDirectRanks; the NS - n surplus loads re-read src[0] (they
+// hit in cache) so that every array element is defined: predicated loads made the compiler keep the packs in
+// scratch.  A destination may be one of the sources (in place): each thread reads a pack before it writes it,
+// and no other thread touches that pack.
 template <int DT, int OP, int NS>
-__device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks], int n, uint64_t dst, int64_t byteOff,
-                                         size_t nbytes, int tid) {
+__device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks], const uint64_t (&dst)[kMaxDirectRanks],
+                                         int n, int64_t byteOff, size_t nbytes, int tid) {
   constexpr int ES = typeSize(DT);
-  uint64_t align = dst | (uint64_t)byteOff;
+  uint64_t align = (uint64_t)byteOff;
 #pragma unroll
-  for (int j = 0; j < NS; j++) align |= src[j];
+  for (int j = 0; j < NS; j++) align |= src[j] | (j < n ? dst[j] : 0);
   size_t doneBytes = 0;
   if ((align & 15u) == 0) {
     const size_t npacks = nbytes >> 4;
@@ -506,7 +520,9 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
 #pragma unroll
       for (int j = 1; j < NS; j++)
         if (j < n) acc = packOp<DT, OP>(acc, v[j]);
-      storePack<false>((char*)dst + byteOff, i, acc);
+#pragma unroll
+      for (int j = 0; j < NS; j++)
+        if (j < n) storePack<false>((char*)dst[j] + byteOff, i, acc);
     }
     doneBytes = npacks << 4;
   }
@@ -517,7 +533,9 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
 #pragma unroll
     for (int j = 1; j < NS; j++)
       if (j < n) acc = wordOp<DT, OP>(acc, loadElem<ES>((const char*)src[j] + byteOff, i));
-    storeElem<ES>((char*)dst + byteOff, i, acc);
+#pragma unroll
+    for (int j = 0; j < NS; j++)
+      if (j < n) storeElem<ES>((char*)dst[j] + byteOff, i, acc);
   }
 }
 
@@ -527,16 +545,16 @@ __device__ __forceinline__ int64_t sweepReal(const SweepGeom& g, int64_t l) {
   return realChunkElems(kAllReduce, g.n, g.C, g.chunkElems, g.alignElems, g.count, grid);
 }
 
-// Phase 0 of the direct all-reduce: for loops [lBegin, lEnd) fold my own chunk from all n send buffers into
-// my receive buffer.  All workgroups sweep the loops together, so at any instant the accesses of the whole
-// grid fall into one window of nChannels * n chunks per buffer.
+// The sweep of the direct all-reduce: for loops [lBegin, lEnd) fold my own chunk from all n send buffers and
+// write the result into all n receive buffers.  All workgroups sweep the loops together, so at any instant the
+// accesses of the whole grid fall into one window of nChannels * n chunks per buffer.
 template <int DT, int OP, int NS>
 __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, int64_t lBegin, int64_t lEnd, int tid) {
   for (int64_t l = lBegin; l < lEnd; l++) {
     const int64_t real = sweepReal(g, l);
     const int64_t off = l * g.loop + ((int64_t)g.ch * g.n + g.me) * real;
     const int64_t nelem = (g.count - off < real) ? g.count - off : real;
-    if (nelem > 0) foldTile<DT, OP, NS>(g.peer, g.n, g.dst, off * g.es, (size_t)(nelem * g.es), tid);
+    if (nelem > 0) foldTile<DT, OP, NS>(g.src, g.dst, g.n, off * g.es, (size_t)(nelem * g.es), tid);
   }
 }
 
@@ -557,12 +575,14 @@ __device__ __forceinline__ void sweepFoldOp(int op, const SweepGeom& g, int64_t 
   }
 }
 
-// The geometry and the buffer table are handed over in LDS and copied to registers here.
+// The geometry and the buffer tables are handed over in LDS and copied to registers here.
 __device__ __forceinline__ void sweepFoldAny(const SweepGeom* gp, int64_t lBegin, int64_t lEnd, int tid) {
   SweepGeom g = *gp;
 #pragma unroll
-  for (int t = 0; t < kMaxDirectRanks; t++) g.peer[t] = uniform64(g.peer[t]);
-  g.dst = uniform64(g.dst);
+  for (int t = 0; t < kMaxDirectRanks; t++) {
+    g.src[t] = uniform64(g.src[t]);
+    g.dst[t] = uniform64(g.dst[t]);
+  }
   const int op = g.op;
   switch (g.dtype) {
     case kF32: sweepFoldOp<kF32>(op, g, lBegin, lEnd, tid); break;
@@ -570,104 +590,6 @@ __device__ __forceinline__ void sweepFoldAny(const SweepGeom* gp, int64_t lBegin
     case kF16: sweepFoldOp<kF16>(op, g, lBegin, lEnd, tid); break;
     case kI32: sweepFoldOp<kI32>(op, g, lBegin, lEnd, tid); break;
     default: sweepFoldOp<kI8>(op, g, lBegin, lEnd, tid); break;
-  }
-}
-
-// Phase 1: for loops [lBegin, lEnd) copy every peer's chunk from that peer's receive buffer into mine.
-__device__ __forceinline__ void sweepGather(const SweepGeom* gp, int64_t lBegin, int64_t lEnd, int tid) {
-  SweepGeom g = *gp;
-#pragma unroll
-  for (int t = 0; t < kMaxDirectRanks; t++) g.peer[t] = uniform64(g.peer[t]);
-  g.dst = uniform64(g.dst);
-  for (int64_t l = lBegin; l < lEnd; l++) {
-    const int64_t real = sweepReal(g, l);
-    const int64_t chunk0 = l * g.loop + (int64_t)g.ch * g.n * real;
-#pragma unroll
-    for (int j = 0; j < kMaxDirectRanks; j++) {
-      if (j >= g.n || j == g.me) continue;
-      const int64_t off = chunk0 + (int64_t)j * real;
-      const int64_t nelem = (g.count - off < real) ? g.count - off : real;
-      if (nelem <= 0) continue;
-      const void* s[1] = {(const char*)g.peer[j] + off * g.es};
-      void* d[1] = {(char*)g.dst + off * g.es};
-      reduceCopyWG<kI8, kSum, 1, 1, kDaemonUnroll, false>(s, d, (size_t)(nelem * g.es), tid, kWgThreads);
-    }
-  }
-}
-
-// One-shot variant: every rank folds the whole (small) message itself.  The owner of a pack, and with it
-// the fold order, follows from the pack's position; the peers' base pointers are read from LDS.
-template <int DT, int OP, int NS>
-__device__ __forceinline__ void foldOneShotN(const uint64_t* peers, int n, char* out, int64_t count, int64_t real,
-                                             int tid) {
-  constexpr int ES = typeSize(DT);
-  constexpr int PACK = 16 / ES;
-  uint64_t align = (uint64_t)(uintptr_t)out;
-#pragma unroll
-  for (int j = 0; j < NS; j++)
-    if (j < n) align |= peers[j];
-  const int64_t npacks = ((align & 15u) == 0) ? (count / PACK) : 0;
-#pragma clang loop vectorize(disable) interleave(disable) unroll(disable)
-  for (int64_t p = tid; p < npacks; p += kWgThreads) {
-    const int owner = (int)((p * PACK) / real);
-    u32x4 v[NS];
-#pragma unroll
-    for (int t = 0; t < NS; t++) {
-      int idx = owner + 1 + (t < n ? t : 0);
-      if (idx >= n) idx -= n;
-      v[t] = loadPack<false>((const char*)peers[idx], (size_t)p);
-    }
-    u32x4 acc = v[0];
-#pragma unroll
-    for (int t = 1; t < NS; t++)
-      if (t < n) acc = packOp<DT, OP>(acc, v[t]);
-    storePack<false>(out, (size_t)p, acc);
-  }
-#pragma clang loop vectorize(disable) interleave(disable) unroll(disable)
-  for (int64_t i = npacks * PACK + tid; i < count; i += kWgThreads) {
-    const int owner = (int)(i / real);
-    int idx = owner + 1;
-    if (idx >= n) idx -= n;
-    uint32_t acc = loadElem<ES>((const char*)peers[idx], (size_t)i);
-#pragma unroll
-    for (int t = 1; t < NS; t++) {
-      if (t < n) {
-        int k = owner + 1 + t;
-        if (k >= n) k -= n;
-        acc = wordOp<DT, OP>(acc, loadElem<ES>((const char*)peers[k], (size_t)i));
-      }
-    }
-    storeElem<ES>(out, (size_t)i, acc);
-  }
-}
-
-template <int DT, int OP>
-__device__ __forceinline__ void foldOneShot(const uint64_t* peers, int n, char* out, int64_t count, int64_t real,
-                                            int tid) {
-  if (n <= 2) foldOneShotN<DT, OP, 2>(peers, n, out, count, real, tid);
-  else if (n <= 4) foldOneShotN<DT, OP, 4>(peers, n, out, count, real, tid);
-  else foldOneShotN<DT, OP, 8>(peers, n, out, count, real, tid);
-}
-
-template <int DT>
-__device__ __forceinline__ void foldOneShotOp(int op, const uint64_t* peers, int n, char* out, int64_t count,
-                                              int64_t real, int tid) {
-  switch (op) {
-    case kSum: foldOneShot<DT, kSum>(peers, n, out, count, real, tid); break;
-    case kProd: foldOneShot<DT, kProd>(peers, n, out, count, real, tid); break;
-    case kMax: foldOneShot<DT, kMax>(peers, n, out, count, real, tid); break;
-    default: foldOneShot<DT, kMin>(peers, n, out, count, real, tid); break;
-  }
-}
-
-__device__ __forceinline__ void foldOneShotAny(int dtype, int op, const uint64_t* peers, int n, char* out,
-                                               int64_t count, int64_t real, int tid) {
-  switch (dtype) {
-    case kF32: foldOneShotOp<kF32>(op, peers, n, out, count, real, tid); break;
-    case kBF16: foldOneShotOp<kBF16>(op, peers, n, out, count, real, tid); break;
-    case kF16: foldOneShotOp<kF16>(op, peers, n, out, count, real, tid); break;
-    case kI32: foldOneShotOp<kI32>(op, peers, n, out, count, real, tid); break;
-    default: foldOneShotOp<kI8>(op, peers, n, out, count, real, tid); break;
   }
 }
 
@@ -763,21 +685,24 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
 
 // ----------------------------------------------------------------- direct protocol
 
-// All-reduce in which the virtual ranks read each other's buffers in place.
+// All-reduce in which the virtual ranks, whose buffers share one HBM, read each
+// other's send buffers and write each other's receive buffers in place.
 // Chunks are laid out as in the FIFO ring (ring_schedule.h): loop l, channel c,
 // chunk j (owned by rank j) starts at l * loop + (c * n + j) * real.
-//   publish   my buffers for this instance; wait until every peer has published;
-//   phase 0   sweep all loops: fold my own chunk from the n send buffers, in the
-//             ring's order for that chunk, into my receive buffer; p1[me] = done;
-//   phase 1   wait until every peer's p1 covers the instance, then sweep all loops
-//             again: copy every peer's chunk from its receive buffer; p2[me] = done;
-//   finally   wait until every peer's p2 covers the instance: nobody reads my
-//             buffers any more, so the completion may be posted.
-// Three waits per instance whatever its size; each is a WaitDesc and can preempt.
-// Messages of at most kOneShotMaxBytes on one channel take a one-shot variant:
-// every rank folds every chunk itself (two waits in total).
-// dyn.step is the phase (2 = only the final wait is left), dyn.gridOffset the
-// next loop of the phase, dyn.slice whether the instance is published.
+//   publish   my buffers for this instance; wait until every peer has published
+//             (its receive buffer may be written from then on);
+//   sweep     all loops: fold my own chunk from the n send buffers, in the ring's
+//             order for that chunk, and store the result into all n receive
+//             buffers; release; p1[me] = loops done;
+//   finally   wait until every peer's p1 covers the instance: every chunk of my
+//             receive buffer has been written and nobody reads my send buffer any
+//             more, so the completion may be posted.
+// Every input element is read once and every output element written once: 2N of
+// traffic per rank for a message of N bytes, against (6n-4)/n * N of the FIFO ring.
+// Two waits per instance whatever its size; each is a WaitDesc and can preempt.
+// dyn.step is the phase (0 = sweep, 2 = only the final wait is left),
+// dyn.gridOffset the next loop of the sweep, dyn.slice whether the instance is
+// published.
 __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
   const CollPlan& P = sh.plan;
   const int lane = tid & 63, wave = tid >> 6;
@@ -792,8 +717,8 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
   const int pubStride = C * (int)sizeof(PeerPub), ctrStride = C * 8;
   const int64_t forceEvery = A.knobs.forceQuitEvery;
   PeerPub* myPub = &P.pubs[(size_t)me * C + ch];
-  int64_t l0 = sh.dyn.gridOffset;
-  int phase = sh.dyn.step;
+  const int64_t l0 = sh.dyn.gridOffset;
+  const int phase = sh.dyn.step;
   __syncthreads();  // every thread has taken its copy of the position before thread 0 changes it
 
   if (!published && tid < 2) {
@@ -804,87 +729,44 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
                        __ATOMIC_RELAXED, DFCCL_AGENT);
     if (tid == 0) sh.dyn.slice = 1;
   }
-  if (!peersLoaded) {
-    // lanes 0..n-1 watch the peers' send words, lanes 32..32+n-1 their receive words
-    const WaitDesc w0 = waitFor(&P.pubs[ch].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
-    const WaitDesc w1 = waitFor(&P.pubs[ch].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
-    if (wave == 0) {
-      const uint64_t word = waitDescs(A, sh, lane, w0, w1, true);
-      if (sh.waitOk && (lane & 31) < n) {
-        if (lane < 32) sh.peerSend[lane] = word & kPtrMask;
-        else sh.peerRecv[lane & 31] = word & kPtrMask;
-      }
-      if (sh.waitOk && lane == 0) sh.peersLoaded = 1;
-    }
-    __syncthreads();
-    if (!sh.waitOk) return kRunPreempted;  // position unchanged
-  }
-
-  if (P.oneShot) {
-    // phase 0: fold everything; then wait until nobody reads any more (in place: via the staging buffer)
-    const int inPlace = (sendbuff == recvbuff);
-    char* out = inPlace ? P.staging + (size_t)me * kOneShotMaxBytes : (char*)recvbuff;
-    if (phase == 0) {
-      const int64_t real = realChunkElems(kAllReduce, n, C, P.chunkElems, P.alignElems, count, 0);
-      if (tid == 0) trace(A, sh, kTrMoveBegin, 0);
-      foldOneShotAny(P.dtype, P.op, sh.peerSend, n, out, count, real, tid);
-      __syncthreads();
-      if (tid == 0) {
-        trace(A, sh, kTrMoveEnd, 0);
-        // released to the system here, while the peers are still busy, so that the completion need not wait for it
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-        if (!inPlace) sh.released = 1;
-        __hip_atomic_store(G(&P.p2[(size_t)me * C + ch]), base + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
-        trace(A, sh, kTrPosted, 2);
-        sh.progressed = 1;
-        sh.slicesSinceLoad++;
-        sh.stats.slicesMoved++;
-      }
-    }
-    const WaitDesc w0 = waitFor(&P.p2[ch], base + 1, ctrStride, n);
-    if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
-    __syncthreads();
-    if (!sh.waitOk) {
-      if (tid == 0) {
-        sh.dyn.gridOffset = 0;
-        sh.dyn.step = 1;
-      }
-      return kRunPreempted;
-    }
-    if (inPlace) {
-      copySlice(out, (void*)recvbuff, nullptr, (size_t)(count * es), tid);
-      __syncthreads();
-    }
-    if (tid == 0) {
-      sh.dyn.instance = inst + 1;
-      sh.dyn.slice = 0;
-    }
-    return kRunDone;
-  }
-
-  if (tid == 0) {
-    SweepGeom& g = sh.sweep;
-    g.count = count;
-    g.loop = loopElems(kAllReduce, n, C, P.chunkElems);
-    g.chunkElems = P.chunkElems;
-    g.alignElems = P.alignElems;
-    g.n = n;
-    g.C = C;
-    g.ch = ch;
-    g.es = es;
-    g.me = me;
-    g.dtype = P.dtype;
-    g.op = P.op;
-    g.pad = 0;
-    g.dst = recvbuff;
-    for (int t = 0; t < kMaxDirectRanks; t++) {
-      if (phase == 0) g.peer[t] = (t < n) ? sh.peerSend[(me + 1 + t) % n] : 0;
-      else g.peer[t] = (t < n) ? sh.peerRecv[t] : 0;
-    }
-  }
-  __syncthreads();
 
   if (phase == 0) {
+    if (!peersLoaded) {
+      // lanes 0..n-1 watch the peers' send words, lanes 32..32+n-1 their receive words
+      const WaitDesc w0 = waitFor(&P.pubs[ch].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
+      const WaitDesc w1 = waitFor(&P.pubs[ch].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
+      if (wave == 0) {
+        const uint64_t word = waitDescs(A, sh, lane, w0, w1, true);
+        if (sh.waitOk && (lane & 31) < n) {
+          // sources in fold order, destinations by rank
+          if (lane < 32) sh.sweep.src[(lane + n - 1 - me) % n] = word & kPtrMask;
+          else sh.sweep.dst[lane & 31] = word & kPtrMask;
+        }
+        if (sh.waitOk && lane >= n && lane < kMaxDirectRanks) {
+          sh.sweep.src[lane] = 0;
+          sh.sweep.dst[lane] = 0;
+        }
+        if (sh.waitOk && lane == 0) {
+          SweepGeom& g = sh.sweep;
+          g.count = count;
+          g.loop = loopElems(kAllReduce, n, C, P.chunkElems);
+          g.chunkElems = P.chunkElems;
+          g.alignElems = P.alignElems;
+          g.n = n;
+          g.C = C;
+          g.ch = ch;
+          g.es = es;
+          g.me = me;
+          g.dtype = P.dtype;
+          g.op = P.op;
+          g.pad = 0;
+          sh.peersLoaded = 1;
+        }
+      }
+      __syncthreads();
+      if (!sh.waitOk) return kRunPreempted;  // position unchanged
+    }
+
     if (tid == 0) trace(A, sh, kTrMoveBegin, 0);
     if (forceEvery > 0) {
       // test hook: one loop at a time, with a preemption point before each
@@ -896,6 +778,8 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
             sh.stats.forcedQuits++;
             sh.dyn.gridOffset = l;
             sh.dyn.step = 0;
+            sh.dyn.wait[0] = noWait();
+            sh.dyn.wait[1] = noWait();
           }
           return kRunPreempted;
         }
@@ -918,70 +802,17 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
     __syncthreads();
     if (tid == 0) {
       trace(A, sh, kTrMoveEnd, 0);
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-      __hip_atomic_store(G(&P.p1[(size_t)me * C + ch]), base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
-      trace(A, sh, kTrPosted, 1);
-      for (int t = 0; t < kMaxDirectRanks; t++) sh.sweep.peer[t] = (t < n) ? sh.peerRecv[t] : 0;
-    }
-    phase = 1;
-    l0 = 0;
-  }
-
-  if (phase == 1) {
-    const WaitDesc w0 = waitFor(&P.p1[ch], base + (uint64_t)L, ctrStride, n);
-    if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
-    __syncthreads();
-    if (!sh.waitOk) {
-      if (tid == 0) {
-        sh.dyn.gridOffset = l0;
-        sh.dyn.step = 1;
-      }
-      return kRunPreempted;
-    }
-    if (tid == 0) trace(A, sh, kTrMoveBegin, 1);
-    if (forceEvery > 0) {
-      for (int64_t l = l0; l < L; l++) {
-        __syncthreads();
-        if (sh.slicesSinceLoad >= forceEvery) {
-          __syncthreads();
-          if (tid == 0) {
-            sh.stats.forcedQuits++;
-            sh.dyn.gridOffset = l;
-            sh.dyn.step = 1;
-            sh.dyn.wait[0] = noWait();
-            sh.dyn.wait[1] = noWait();
-          }
-          return kRunPreempted;
-        }
-        __syncthreads();
-        sweepGather(&sh.sweep, l, l + 1, tid);
-        if (tid == 0) {
-          sh.progressed = 1;
-          sh.slicesSinceLoad++;
-          sh.stats.slicesMoved++;
-        }
-      }
-    } else {
-      sweepGather(&sh.sweep, l0, L, tid);
-      if (tid == 0) {
-        sh.progressed = 1;
-        sh.slicesSinceLoad += L - l0;
-        sh.stats.slicesMoved += (uint64_t)(L - l0);
-      }
-    }
-    __syncthreads();
-    if (tid == 0) {
-      trace(A, sh, kTrMoveEnd, 1);
+      // released to the system here, while the peers are still busy, so that the completion need not wait for it
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
       sh.released = 1;
-      __hip_atomic_store(G(&P.p2[(size_t)me * C + ch]), base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
-      trace(A, sh, kTrPosted, 2);
+      __hip_atomic_store(G(&P.p1[(size_t)me * C + ch]), base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
+      trace(A, sh, kTrPosted, 1);
     }
   }
 
-  // nobody may still be reading my send buffer or my chunks of the receive buffer
+  // every chunk of my receive buffer is written, and nobody reads my send buffer any more
   {
-    const WaitDesc w0 = waitFor(&P.p2[ch], base + (uint64_t)L, ctrStride, n);
+    const WaitDesc w0 = waitFor(&P.p1[ch], base + (uint64_t)L, ctrStride, n);
     if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
     __syncthreads();
     if (!sh.waitOk) {
@@ -1030,7 +861,6 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
     sh.slicesSinceLoad = 0;
     sh.dyn.wait[0] = noWait();
     sh.dyn.wait[1] = noWait();
-    sh.statsDirty = 1;
     trace(A, sh, kTrVisitBegin, coll);
   }
   __syncthreads();
@@ -1061,9 +891,9 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
         // a rank with a single channel has a single poster, which keeps the ticket itself
         const uint64_t t = (R.nChannels == 1) ? sh.cqNext++
                                               : __hip_atomic_fetch_add(G(R.cqTicket), 1ull, __ATOMIC_RELAXED, DFCCL_AGENT);
-        __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]),
-                           cqeEncode((unsigned)ch, (unsigned)(t + 1), (unsigned)sh.plan.collId), __ATOMIC_RELEASE,
-                           DFCCL_SYSTEM);
+        const uint64_t cqe = cqeEncode((unsigned)ch, (unsigned)(t + 1), (unsigned)sh.plan.collId);
+        if (sh.released) __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]), cqe, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+        else __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]), cqe, __ATOMIC_RELEASE, DFCCL_SYSTEM);
         sh.stats.cqesWritten++;
         trace(A, sh, kTrCqePosted, coll);
       }
@@ -1082,8 +912,10 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
   __shared__ WgShared sh;
   const DaemonArgs& A = *argsPtr;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // Workgroups go to the XCDs round robin.  The channels of a rank are rotated by its slot, so that the
+  // leaders (channel 0), which talk to the host, do not all sit on one XCD.
   const int slot = (int)blockIdx.x / A.channelsPerRank;
-  const int ch = (int)blockIdx.x % A.channelsPerRank;
+  const int ch = ((int)blockIdx.x % A.channelsPerRank + A.channelsPerRank - slot % A.channelsPerRank) % A.channelsPerRank;
   if (slot >= A.nSlots) return;
   const RankDev& R = A.ranks[slot];
   if (!R.active || ch >= R.nChannels) return;
@@ -1105,10 +937,11 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     sh.progressedRound = 0;
     sh.loadedColl = -1;
     sh.peersLoaded = 0;
-    sh.wgIndex = blockIdx.x;
+    sh.wgIndex = (uint32_t)(slot * A.channelsPerRank + ch);
     sh.traceCount = 0;
     sh.round = 0;
     sh.allFresh = 0;
+    sh.rankBusy = 0;
     sh.cqNext = S.cqNext;
     trace(A, sh, kTrLaunch, A.epoch);
     const DFCCL_GLOBAL WgStats* hs = G(&R.stats[ch]);
@@ -1120,7 +953,8 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     sh.stats.forcedQuits = hs->forcedQuits;
     sh.stats.slicesMoved = hs->slicesMoved;
     sh.stats.spins = hs->spins;
-    sh.statsDirty = 0;
+    sh.statsEpoch = 0;
+    sh.statsReqSeen = 0;
   }
   __syncthreads();
   for (int i = tid; i < sh.numActive; i += kWgThreads) sh.taskq[i] = S.taskq[i];
@@ -1141,6 +975,12 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
         if ((sh.round++ & 7u) == 0) {
           abortFlag = __hip_atomic_load(G(&A.devFlags[1]), __ATOMIC_RELAXED, DFCCL_AGENT);
           quitFlag = __hip_atomic_load(G(&A.devFlags[0]), __ATOMIC_RELAXED, DFCCL_AGENT);
+          const uint32_t statsReq = __hip_atomic_load(G(&A.devFlags[2]), __ATOMIC_RELAXED, DFCCL_AGENT);
+          if (statsReq != sh.statsEpoch) {
+            // the host wants the counters
+            sh.statsEpoch = statsReq;
+            flushStats(R, sh, ch, statsReq);
+          }
           expired = K.maxLifetimeTicks > 0 && (int64_t)(wall_clock64() - startTick) > K.maxLifetimeTicks;
         }
         if (sh.ingested > 0 || sh.progressedRound) sh.idle = 0;
@@ -1150,12 +990,11 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
         else if (quitFlag || expired) sh.exitKind = kExitVoluntary;
         else if (sh.idle >= K.tolerantUnprogressedCnt) sh.exitKind = kExitVoluntary;
         sh.progressedRound = 0;
-        // counters go to the host when the workgroup has nothing better to do
-        if (sh.numReady == 0 && sh.statsDirty) flushStats(R, sh, ch);
       }
       if (sh.numReady == 0 && sh.ingested == 0) {
         // nothing can move: the leader's next poll is a PCIe round trip anyway, the others back off a little
         if (ch != 0) __builtin_amdgcn_s_sleep(20);
+        else if (sh.rankBusy) __builtin_amdgcn_s_sleep(100);
       }
     }
     __syncthreads();
@@ -1209,7 +1048,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     trace(A, sh, kTrExit, (uint32_t)exitKind);
     if (A.trace != nullptr)  // the last record slot of the workgroup holds how many records it wrote
       G(A.trace)[((size_t)sh.wgIndex * kTraceRecords + (kTraceRecords - 1)) * 2 + 1] = sh.traceCount;
-    flushStats(R, sh, ch);
+    flushStats(R, sh, ch, sh.statsEpoch);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
     __hip_atomic_store(G(&R.wgExit[ch]), (A.epoch << 4) | (uint32_t)exitKind, __ATOMIC_RELEASE, DFCCL_SYSTEM);
   }

@@ -96,7 +96,6 @@ DFCCL_HD bool waitReached(uint64_t word, uint64_t value, bool tagged) {
 
 enum Proto : int { kProtoFifo = 0, kProtoDirect = 1 };
 constexpr int kMaxDirectRanks = 8;           // ranks whose buffers one workgroup folds in a single pass
-constexpr int kOneShotMaxBytes = 32 << 10;  // 512 threads x 4 packs of 16 bytes
 
 // Immutable plan of one collective on one rank (HBM, written at finalize).
 struct alignas(16) CollPlan {
@@ -116,11 +115,9 @@ struct alignas(16) CollPlan {
   ConnFlags* recvFlags;
   uint64_t* doneCounter;   // workgroups that finished an instance, monotonic
   // direct protocol (peers read each other's buffers, no FIFO)
-  int32_t proto, oneShot;
+  int32_t proto, pad2;
   PeerPub* pubs;           // [nRanks][nChannels]
-  uint64_t* p1;            // [nRanks][nChannels] loops whose own chunk is reduced and stored
-  uint64_t* p2;            // [nRanks][nChannels] loops whose reads of peer buffers are finished
-  char* staging;           // one-shot, in place: kOneShotMaxBytes per rank
+  uint64_t* p1;            // [nRanks][nChannels] loops whose own chunk is folded and stored everywhere
   int64_t loopsPerInstance;
 };
 
@@ -141,10 +138,14 @@ struct alignas(128) DynCtx {
   uint64_t pad[2];
 };
 
-// Counters of one workgroup, in host-coherent memory so the host can read them
-// while the daemon runs.
-struct alignas(64) WgStats {
+// Counters of one workgroup, in host-coherent memory.  A workgroup writes them when it leaves the kernel, and
+// when the host asks (the host raises the request number in the word after the control word; a workgroup that
+// has written its counters for request e stores e in `epoch`).  They are not written after every collective:
+// thousands of small writes over PCIe would queue up in front of the completions.
+struct alignas(128) WgStats {
   uint64_t sqesRead, cqesWritten, ctxSaves, ctxLoads, voluntaryQuits, forcedQuits, slicesMoved, spins;
+  uint64_t epoch;
+  uint64_t pad[7];
 };
 
 // Scheduler state a workgroup saves when it leaves voluntarily and restores at
@@ -190,6 +191,7 @@ struct Knobs {
   int64_t tolerantUnprogressedCnt;  // TOLERANT_UNPROGRESSED_CNT, default 500000
   int64_t forceQuitEvery;           // DFCCL_FORCE_QUIT_EVERY: preempt after this many slices (0 = off)
   int64_t maxLifetimeTicks;         // DFCCL_DAEMON_MAX_MS in 100 MHz ticks (0 = unlimited)
+  int64_t idlePollRounds;           // DFCCL_IDLE_POLL_ROUNDS: x 4 pipelined polls per idle round of a leader (0 = off)
 };
 
 struct DaemonArgs {

@@ -92,12 +92,10 @@ struct CommGroup {
   char* fifo = nullptr;
   ConnFlags* flags = nullptr;
   // direct protocol
-  int proto = kProtoFifo, oneShot = 0;
+  int proto = kProtoFifo;
   int64_t loopsPerInstance = 0;
   PeerPub* pubs = nullptr;   // [nRanks][nChannels]
   uint64_t* p1 = nullptr;    // [nRanks][nChannels]
-  uint64_t* p2 = nullptr;
-  char* staging = nullptr;   // [nRanks][kOneShotMaxBytes], one-shot only
 };
 
 }  // namespace dfccl
@@ -171,7 +169,8 @@ struct Daemon {
   uint32_t epoch = 0;
   uint64_t launches = 0;
   long capacity = 0;
-  uint32_t* ctrl = nullptr;      // host-coherent
+  uint32_t* ctrl = nullptr;      // host-coherent: [0] control word, [1] request number for the counters
+  uint32_t statsEpoch = 0;
   uint32_t* devFlags = nullptr;  // HBM
   DaemonArgs* devArgs = nullptr; // HBM
   DaemonArgs hostArgs{};
@@ -214,6 +213,7 @@ struct Daemon {
     knobs.tolerantUnprogressedCnt = envInt("TOLERANT_UNPROGRESSED_CNT", 500000);
     knobs.forceQuitEvery = envInt("DFCCL_FORCE_QUIT_EVERY", 0);
     knobs.maxLifetimeTicks = envInt("DFCCL_DAEMON_MAX_MS", 0) * 100000;  // wall_clock64 runs at 100 MHz
+    knobs.idlePollRounds = envInt("DFCCL_IDLE_POLL_ROUNDS", 8);
     if (knobs.numTryTaskqHead < 1) knobs.numTryTaskqHead = 1;
     if (knobs.tolerantUnprogressedCnt < 1) knobs.tolerantUnprogressedCnt = 1;
   }
@@ -324,7 +324,7 @@ static ncclResult_t getDaemon(int device, Daemon** out) {
   HIPCHECK(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
   HIPCHECK(hipEventCreateWithFlags(&d->doneEv, hipEventBlockingSync | hipEventDisableTiming));
   HIPCHECK(hipHostMalloc((void**)&d->ctrl, 64, hipHostMallocCoherent | hipHostMallocMapped));
-  *d->ctrl = 0;
+  memset(d->ctrl, 0, 64);
   HIPCHECK(hipMalloc((void**)&d->devFlags, 64));
   HIPCHECK(hipMemset(d->devFlags, 0, 64));
   HIPCHECK(hipMalloc((void**)&d->devArgs, sizeof(DaemonArgs)));
@@ -448,10 +448,6 @@ static void planGroup(CommGroup* g) {
   g->chanStride = g->slotBytes * g->fifoSlots;
   const int64_t loop = loopElems(g->kind, g->nRanks, g->nChannels, g->chunkElems);
   g->loopsPerInstance = g->count > 0 ? divUp64(g->count, loop) : 0;
-  g->oneShot = (g->proto == kProtoDirect && g->nChannels == 1 && g->loopsPerInstance <= 1 &&
-                g->count * g->elemSize <= kOneShotMaxBytes && envInt("DFCCL_ONESHOT", 1) != 0)
-                   ? 1
-                   : 0;
 }
 
 static ncclResult_t allocGroupLocked(CommGroup* g) {
@@ -466,9 +462,6 @@ static ncclResult_t allocGroupLocked(CommGroup* g) {
     HIPCHECK(hipMemset(g->pubs, 0, links * sizeof(PeerPub)));
     HIPCHECK(hipMalloc((void**)&g->p1, links * 8));
     HIPCHECK(hipMemset(g->p1, 0, links * 8));
-    HIPCHECK(hipMalloc((void**)&g->p2, links * 8));
-    HIPCHECK(hipMemset(g->p2, 0, links * 8));
-    if (g->oneShot) HIPCHECK(hipMalloc((void**)&g->staging, (size_t)g->nRanks * kOneShotMaxBytes));
   }
   return ncclSuccess;
 }
@@ -676,12 +669,12 @@ DFCCL_API ncclResult_t ncclCommDestroy(ncclComm_t comm) {
     if (d != nullptr) {
       std::lock_guard<std::mutex> lk(d->mu);
       if (d->running) {
-        for (void* p : {(void*)g->fifo, (void*)g->flags, (void*)g->pubs, (void*)g->p1, (void*)g->p2, (void*)g->staging})
+        for (void* p : {(void*)g->fifo, (void*)g->flags, (void*)g->pubs, (void*)g->p1})
           if (p) d->garbageDev.push_back(p);
-        g->fifo = nullptr; g->flags = nullptr; g->pubs = nullptr; g->p1 = nullptr; g->p2 = nullptr; g->staging = nullptr;
+        g->fifo = nullptr; g->flags = nullptr; g->pubs = nullptr; g->p1 = nullptr;
       }
     }
-    for (void* p : {(void*)g->fifo, (void*)g->flags, (void*)g->pubs, (void*)g->p1, (void*)g->p2, (void*)g->staging})
+    for (void* p : {(void*)g->fifo, (void*)g->flags, (void*)g->pubs, (void*)g->p1})
       if (p) (void)hipFree(p);
     delete g;
   }
@@ -789,8 +782,8 @@ DFCCL_API ncclResult_t ofcclFinalizeRankCtx7StartHostThrds(ofcclRankCtx_t c) {
     p.slotBytes = g->slotBytes; p.fifoChanStride = g->chanStride;
     p.sendFifo = g->fifo ? g->fifo + (size_t)rank * g->nChannels * g->chanStride : nullptr;
     p.recvFifo = g->fifo ? g->fifo + (size_t)prev * g->nChannels * g->chanStride : nullptr;
-    p.proto = g->proto; p.oneShot = g->oneShot; p.pubs = g->pubs; p.p1 = g->p1; p.p2 = g->p2;
-    p.staging = g->staging; p.loopsPerInstance = g->loopsPerInstance;
+    p.proto = g->proto; p.pad2 = 0; p.pubs = g->pubs; p.p1 = g->p1;
+    p.loopsPerInstance = g->loopsPerInstance;
     p.sendFlags = g->flags + (size_t)rank * g->nChannels;
     p.recvFlags = g->flags + (size_t)prev * g->nChannels;
     p.doneCounter = c->doneCounters + i;
@@ -968,6 +961,31 @@ DFCCL_API ncclResult_t dfcclGetStats(ofcclRankCtx_t c, dfcclStats* out) {
   if (c == nullptr || out == nullptr) return ncclInvalidArgument;
   memset(out, 0, sizeof(*out));
   if (!c->finalized) return ncclInvalidUsage;
+  Daemon* d = c->daemon;
+  {
+    // A resident daemon writes its counters on request: raise the request number (the word after the control
+    // word) and wait, for a bounded time, until every workgroup of this rank has answered. Workgroups in the
+    // middle of a long transfer answer late; then the figures are those of their previous answer.
+    std::unique_lock<std::mutex> lk(d->mu);
+    if (d->running && !d->failed) {
+      uint32_t e = ++d->statsEpoch;
+      if (e == 0) e = ++d->statsEpoch;
+      __atomic_store_n(&d->ctrl[1], e, __ATOMIC_RELEASE);
+      lk.unlock();
+      const uint64_t deadline = nowNs() + 20000000ull;
+      for (;;) {
+        bool all = true;
+        for (int ch = 0; ch < c->nChannels && all; ch++)
+          all = __atomic_load_n(&c->dev.stats[ch].epoch, __ATOMIC_ACQUIRE) == (uint64_t)e;
+        if (all || nowNs() > deadline) break;
+        lk.lock();
+        const bool gone = !d->running;
+        lk.unlock();
+        if (gone) break;
+        usleep(20);
+      }
+    }
+  }
   for (int ch = 0; ch < c->nChannels; ch++) {
     const WgStats* s = &c->dev.stats[ch];
     out->sqesRead += __atomic_load_n(&s->sqesRead, __ATOMIC_ACQUIRE);
@@ -978,8 +996,8 @@ DFCCL_API ncclResult_t dfcclGetStats(ofcclRankCtx_t c, dfcclStats* out) {
     out->forcedQuits += __atomic_load_n(&s->forcedQuits, __ATOMIC_ACQUIRE);
     out->slicesMoved += __atomic_load_n(&s->slicesMoved, __ATOMIC_ACQUIRE);
   }
-  std::lock_guard<std::mutex> lk(c->daemon->mu);
-  out->daemonLaunches = c->daemon->launches;
+  std::lock_guard<std::mutex> lk(d->mu);
+  out->daemonLaunches = d->launches;
   return ncclSuccess;
 }
 
@@ -1002,6 +1020,5 @@ DFCCL_API ncclResult_t dfcclGetCollGeometry(ofcclRankCtx_t c, int collId, dfcclC
   geom->slicesPerChunk = g->slicesPerChunk;
   geom->fifoSlots = g->fifoSlots;
   geom->protocol = g->proto;
-  geom->oneShot = g->oneShot;
   return ncclSuccess;
 }

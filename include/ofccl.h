@@ -189,7 +189,6 @@ typedef struct {
   int slicesPerChunk;
   int fifoSlots;
   int protocol;        /* 0: FIFO ring, 1: direct (peers read each other's buffers) */
-  int oneShot;         /* direct protocol, message small enough for the two-exchange variant */
 } dfcclCollGeometry;
 ncclResult_t dfcclGetCollGeometry(ofcclRankCtx_t rankCtx, int collId, dfcclCollGeometry* geom);
 

@@ -74,9 +74,9 @@ def test_config5_preemption_under_gemm_contention(proto, monkeypatch):
     monkeypatch.setenv("DFCCL_PROTO", proto)
     monkeypatch.setenv("DFCCL_DAEMON_MAX_MS", "20000")
     results = {}
-    # a FIFO channel of this collective moves 15 steps x 2 slices of 256 KiB in all, fewer than 64: there the
-    # hook fires every 8 slices instead, so that every workgroup is preempted several times per collective
-    forced = "64" if proto == "direct" else "8"
+    # a workgroup moves 32 slices (direct: one 16 KiB chunk per loop) or 30 slices (FIFO: 15 steps x 2 slices of
+    # 256 KiB) per collective here: the hook fires every 8 slices, so every workgroup is preempted several times
+    forced = "8"
     for force in ("0", forced):
         monkeypatch.setenv("DFCCL_FORCE_QUIT_EVERY", force)
         frecv = [torch.zeros_like(t) for t in fsend]

@@ -359,15 +359,12 @@ def test_prepare_validation_follows_the_reference():
 
 @pytest.mark.parametrize("dtype,op", [(orc.F16, orc.SUM), (orc.BF16, orc.SUM), (orc.F32, orc.PROD), (orc.I8, orc.MAX)])
 @pytest.mark.parametrize("n,count", [(4, 2048), (2, 1), (8, 16384 // 4), (3, 1000), (5, 8191)])
-def test_small_all_reduce_one_shot_and_in_place(dtype, op, n, count, proto):
-    # small messages take the one-shot variant of the direct protocol; in place goes through staging
+def test_small_all_reduce_and_in_place(dtype, op, n, count, proto):
+    # small messages (some ranks own no chunk at all), out of place and in place
     from dfccl_amd.ring import VirtualRing
     with VirtualRing(n) as ring:
         ring.prepare(0, "all_reduce", count, dtype, op)
         ring.finalize()
-        g = ring.ctxs[0].geometry(0)
-        if proto == "direct" and count * orc.TYPE_SIZE[dtype] <= 32768:
-            assert g.oneShot == 1
         sends_np, sends, recvs = make_buffers("all_reduce", dtype, n, count, 1100, small_ints=(op == orc.PROD))
         want = orc.all_reduce(dtype, op, geom_of(ring, 0), sends_np)
         for rep in range(3):
@@ -381,7 +378,7 @@ def test_small_all_reduce_one_shot_and_in_place(dtype, op, n, count, proto):
             assert np.array_equal(to_np(dtype, bufs[r]), want[r]), ("in place", r)
 
 
-def test_one_shot_under_forced_preemption(monkeypatch):
+def test_small_all_reduce_under_forced_preemption(monkeypatch):
     monkeypatch.setenv("DFCCL_FORCE_QUIT_EVERY", "1")
     check("all_reduce", orc.F32, orc.SUM, 4, 1024, seed=1200, reps=3)
     monkeypatch.setenv("BASE_CTX_SWITCH_THRESHOLD", "1")
