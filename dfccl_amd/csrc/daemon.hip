@@ -35,12 +35,14 @@ namespace dfccl {
 
 constexpr int kDaemonUnroll = 1;  // see reduce_copy.hip: shallow unrolling keeps DRAM accesses ordered
 constexpr int kReadyWords = (kMaxColls + 63) / 64;
+constexpr int kExpressMaxBytes = 4096;  // largest own chunk wave 0 folds by itself (see runExpress)
+constexpr int kIdleRounds = 8;  // x 4 polls of the host ring before an idle leader goes round its main loop again
 enum RunStatus : int { kRunDone = 0, kRunPreempted = 1 };
 
 // Geometry of the direct all-reduce sweeps: loop l covers elements [l * loop, (l + 1) * loop), split into
 // nChannels * n chunks of `real` elements; every loop but the last uses the nominal chunk.
 struct SweepGeom {
-  int64_t count, loop, chunkElems, alignElems;
+  int64_t count, loop, chunkElems, lastReal, L;
   int n, C, ch, es;
   int me, dtype, op, pad;
   uint64_t src[kMaxDirectRanks];     // the send buffers in fold order: in[me + 1], in[me + 2], ..., in[me]
@@ -64,6 +66,7 @@ struct WgShared {
   uint32_t traceCount;
   uint32_t wgIndex;
   uint32_t round;          // scheduler rounds since launch
+  int32_t express;         // the submission just ingested qualifies for the express path
   int32_t rankBusy;        // leader: other channels of the rank still have work in flight
   int32_t allFresh;        // every collective of the task queue was ingested this round (nothing is parked)
   uint64_t cqNext;         // single-channel ranks: next completion ticket
@@ -178,6 +181,7 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
   const uint64_t mm = __ballot(mine && lane < take);
   const int pos = __builtin_popcountll(mm & ((1ull << lane) - 1ull));
   const int base = sh.numActive;
+  bool expressLane = false;
   if (mine && lane < take && base + pos < kMaxColls) {
     DFCCL_GLOBAL DynCtx* d = G(&R.dyn[(size_t)ch * R.nColls + coll]);
     d->sendbuff = sendbuff;
@@ -189,9 +193,23 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
       sh.dyn.recvbuff = recvbuff;
       sh.dyn.active = 1;
       sh.peersLoaded = 0;
+      if (sh.plan.proto == kProtoDirect && sh.dyn.slice == 0) {
+        // and tell the peers at once where its buffers are, instead of when the scheduler gets to it
+        PeerPub* myPub = &sh.plan.pubs[(size_t)sh.plan.rank * sh.plan.nChannels + ch];
+        const uint64_t tag = pubTag(sh.dyn.instance);
+        __hip_atomic_store(G(&myPub->send), sendbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
+        __hip_atomic_store(G(&myPub->recv), recvbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
+        sh.dyn.slice = 1;
+        // alone in the queue and small: wave 0 can run it on the spot (see runExpress)
+        if (base == 0 && __builtin_popcountll(mm) == 1 && sh.plan.nChannels == 1 && sh.plan.loopsPerInstance == 1 &&
+            sh.plan.lastChunkElems * sh.plan.elemSize <= kExpressMaxBytes && A.knobs.forceQuitEvery == 0 &&
+            A.knobs.express != 0 && sh.dyn.step == 0)
+          expressLane = true;
+      }
     }
     sh.taskq[base + pos] = (uint16_t)coll;
   }
+  const bool express = __ballot(expressLane) != 0;
   if (lane == 0) {
     const int added = __builtin_popcountll(mm);
     sh.numActive = base + added;
@@ -200,6 +218,7 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
     if (q < avail) sh.finalQuit = 1;
     sh.ingested = consumed;
     sh.allFresh = (base == 0) ? 1 : 0;
+    sh.express = express ? 1 : 0;
     sh.stats.sqesRead += (uint64_t)consumed;
     if (R.nChannels > 1) __hip_atomic_store(G(&R.wgFrontier[ch]), sh.frontier, __ATOMIC_RELAXED, DFCCL_AGENT);
     trace(A, sh, kTrIngested, (uint32_t)consumed);
@@ -255,7 +274,10 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
     __builtin_amdgcn_s_sleep(2);                                                                              \
     q = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_SYSTEM);                                                 \
   }
-    for (int it = 0; it < idleRounds; it++) {
+    // the trip count is a constant on purpose: the unrolled loop keeps its four loads in flight, a rolled one
+    // waits for all of them at its head
+#pragma unroll
+    for (int it = 0; it < kIdleRounds; it++) {
       DFCCL_IDLE_STEP(q0)
       DFCCL_IDLE_STEP(q1)
       DFCCL_IDLE_STEP(q2)
@@ -540,9 +562,7 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
 }
 
 __device__ __forceinline__ int64_t sweepReal(const SweepGeom& g, int64_t l) {
-  const int64_t grid = l * g.loop;
-  if (g.count - grid >= g.loop) return g.chunkElems;
-  return realChunkElems(kAllReduce, g.n, g.C, g.chunkElems, g.alignElems, g.count, grid);
+  return (l == g.L - 1) ? g.lastReal : g.chunkElems;
 }
 
 // The sweep of the direct all-reduce: for loops [lBegin, lEnd) fold my own chunk from all n send buffers and
@@ -751,7 +771,8 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
           g.count = count;
           g.loop = loopElems(kAllReduce, n, C, P.chunkElems);
           g.chunkElems = P.chunkElems;
-          g.alignElems = P.alignElems;
+          g.lastReal = P.lastChunkElems;
+          g.L = L;
           g.n = n;
           g.C = C;
           g.ch = ch;
@@ -811,6 +832,7 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
   }
 
   // every chunk of my receive buffer is written, and nobody reads my send buffer any more
+  if (phase != 0 && tid == 0) sh.released = 1;  // resumed here: the sweep's release was done before it was parked
   {
     const WaitDesc w0 = waitFor(&P.p1[ch], base + (uint64_t)L, ctrStride, n);
     if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
@@ -833,6 +855,152 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
 __device__ __forceinline__ int runColl(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
   if (sh.plan.proto == kProtoDirect) return runDirectAllReduce(A, sh, ch, tid);
   return runFifo(A, sh, ch, tid);
+}
+
+// One thread: the resident collective has finished an instance.  Resets its position for the next instance
+// (link counters and the instance number persist), posts the completion and stores the context.
+// (manipulateCQ7ResetDoneColl, enqueue_ofccl_dev.cu:773-920.)
+__device__ __forceinline__ void completeColl(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, uint32_t coll) {
+  sh.dyn.gridOffset = 0;
+  sh.dyn.step = 0;
+  sh.dyn.tryCnt = 0;
+  sh.dyn.active = 0;
+  if (sh.plan.proto == kProtoFifo) sh.dyn.slice = 0;
+  sh.dyn.wait[0] = noWait();
+  sh.dyn.wait[1] = noWait();
+  sh.peersLoaded = 0;
+  // results are released to the system (unless the protocol has done so already), then the last channel to
+  // finish posts the entry
+  if (!sh.released) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+  bool last = true;
+  if (sh.plan.nChannels > 1) {
+    const uint64_t old = __hip_atomic_fetch_add(G(sh.plan.doneCounter), 1ull, __ATOMIC_ACQ_REL, DFCCL_AGENT);
+    last = ((old + 1) % (uint64_t)sh.plan.nChannels == 0);
+  }
+  if (last) {
+    // a rank with a single channel has a single poster, which keeps the ticket itself
+    const uint64_t t = (R.nChannels == 1) ? sh.cqNext++
+                                          : __hip_atomic_fetch_add(G(R.cqTicket), 1ull, __ATOMIC_RELAXED, DFCCL_AGENT);
+    const uint64_t cqe = cqeEncode((unsigned)ch, (unsigned)(t + 1), (unsigned)sh.plan.collId);
+    if (sh.released) __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]), cqe, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+    else __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]), cqe, __ATOMIC_RELEASE, DFCCL_SYSTEM);
+    sh.stats.cqesWritten++;
+    trace(A, sh, kTrCqePosted, coll);
+  }
+  storeStruct(&R.dyn[(size_t)ch * R.nColls + coll], sh.dyn);
+}
+
+template <int DT>
+__device__ __forceinline__ u32x4 foldPacksOp(int op, const u32x4 (&v)[kMaxDirectRanks], int n) {
+  u32x4 acc = v[0];
+#pragma unroll
+  for (int t = 1; t < kMaxDirectRanks; t++) {
+    if (t < n) {
+      switch (op) {
+        case kSum: acc = packOp<DT, kSum>(acc, v[t]); break;
+        case kProd: acc = packOp<DT, kProd>(acc, v[t]); break;
+        case kMax: acc = packOp<DT, kMax>(acc, v[t]); break;
+        default: acc = packOp<DT, kMin>(acc, v[t]); break;
+      }
+    }
+  }
+  return acc;
+}
+
+// The express path for small all-reduces, run by wave 0 alone inside the ingest phase: when the submission
+// that just arrived is the only work of the workgroup, is the next instance of the resident collective (so
+// its buffers have been published at ingest already), uses the direct protocol on one channel in one loop
+// and this rank's chunk is at most kExpressMaxBytes, the wave does the whole instance (wait for the peers'
+// buffers, fold, store everywhere, release, wait for the peers, post the completion) without a workgroup
+// barrier and without going through the scheduler.  A wait that runs out of budget, or buffers that are not
+// 16-byte aligned, hand the collective to the scheduler in the state it has reached.  Returns true if the
+// instance is complete.
+__device__ __forceinline__ bool runExpress(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane) {
+  const CollPlan& P = sh.plan;
+  const uint32_t coll = sh.taskq[0];
+  const int n = P.nRanks, es = P.elemSize, me = P.rank;
+  const uint64_t inst = sh.dyn.instance;
+  const int pubStride = (int)sizeof(PeerPub);  // one channel
+  if (lane == 0) {
+    sh.threshold = A.knobs.baseCtxSwitchThreshold * A.knobs.numTryTaskqHead;
+    if (sh.threshold < 1) sh.threshold = 1;
+    sh.waitOk = 1;
+    sh.released = 0;
+    sh.slicesSinceLoad = 0;
+    trace(A, sh, kTrVisitBegin, coll);
+  }
+  // lanes 0..n-1 get the peers' send buffers, lanes 32..32+n-1 their receive buffers
+  const WaitDesc w0 = waitFor(&P.pubs[0].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
+  const WaitDesc w1 = waitFor(&P.pubs[0].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
+  const uint64_t word = waitDescs(A, sh, lane, w0, w1, false) & kPtrMask;
+  if (!sh.waitOk) return false;  // nothing done yet: the scheduler starts from the published state
+  const int64_t real = P.lastChunkElems;
+  const int64_t off = (int64_t)me * real;
+  int64_t nelem = (P.count - off < real) ? P.count - off : real;
+  if (nelem < 0) nelem = 0;
+  const int64_t byteOff = off * es;
+  const size_t nbytes = (size_t)(nelem * es);
+  // every pointer and the length must allow 128-bit accesses
+  uint64_t misaligned = ((lane & 31) < n) ? (word & 15u) : 0;
+  misaligned |= (uint64_t)(nbytes & 15u);
+  if (__ballot(misaligned != 0) != 0) return false;
+  if (lane == 0) trace(A, sh, kTrMoveBegin, 0);
+  uint64_t src[kMaxDirectRanks], dst[kMaxDirectRanks];
+#pragma unroll
+  for (int t = 0; t < kMaxDirectRanks; t++) {
+    int r = me + 1 + t;  // fold order in[me + 1], in[me + 2], ..., in[me]; surplus entries repeat the first
+    if (t >= n) r = me + 1;
+    if (r >= n) r -= n;
+    src[t] = uniform64(__shfl(word, r));
+    dst[t] = uniform64(__shfl(word, 32 + (t < n ? t : 0)));
+  }
+  const size_t npacks = nbytes >> 4;
+  for (size_t i = lane; i < npacks; i += 64) {
+    u32x4 v[kMaxDirectRanks];
+#pragma unroll
+    for (int t = 0; t < kMaxDirectRanks; t++) v[t] = loadPack<true>((const char*)src[t] + byteOff, i);
+    u32x4 acc;
+    switch (P.dtype) {
+      case kF32: acc = foldPacksOp<kF32>(P.op, v, n); break;
+      case kBF16: acc = foldPacksOp<kBF16>(P.op, v, n); break;
+      case kF16: acc = foldPacksOp<kF16>(P.op, v, n); break;
+      case kI32: acc = foldPacksOp<kI32>(P.op, v, n); break;
+      default: acc = foldPacksOp<kI8>(P.op, v, n); break;
+    }
+#pragma unroll
+    for (int t = 0; t < kMaxDirectRanks; t++)
+      if (t < n) storePack<false>((char*)dst[t] + byteOff, i, acc);
+  }
+  // all lanes' stores are covered by the wave's release
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+  if (lane == 0) {
+    trace(A, sh, kTrMoveEnd, 0);
+    sh.released = 1;
+    __hip_atomic_store(G(&P.p1[me]), inst + 1, __ATOMIC_RELAXED, DFCCL_AGENT);  // one loop per instance
+    trace(A, sh, kTrPosted, 1);
+    sh.progressedRound = 1;
+    sh.stats.slicesMoved++;
+  }
+  const WaitDesc wp = waitFor(&P.p1[0], inst + 1, 8, n);
+  waitDescs(A, sh, lane, wp, noWait(), false);
+  if (!sh.waitOk) {
+    // the scheduler takes over at the final wait (waitDescs has stored what the collective is parked on)
+    if (lane == 0) {
+      sh.dyn.gridOffset = 0;
+      sh.dyn.step = 2;
+      sh.stats.ctxSaves++;
+      storeStruct(&R.dyn[(size_t)ch * R.nColls + coll], sh.dyn);
+    }
+    return false;
+  }
+  if (lane == 0) {
+    sh.dyn.instance = inst + 1;
+    sh.dyn.slice = 0;
+    completeColl(A, R, sh, ch, coll);
+    sh.numActive = 0;
+    trace(A, sh, kTrVisitEnd, 0);
+  }
+  return true;
 }
 
 // Visit one collective of the task queue: make its context resident, run it,
@@ -869,35 +1037,8 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
   if (tid == 0) {
     if (sh.progressed) sh.progressedRound = 1;
     if (status == kRunDone) {
-      // reset the position for the next instance; link counters and the instance number persist
-      sh.dyn.gridOffset = 0;
-      sh.dyn.step = 0;
-      sh.dyn.tryCnt = 0;
-      sh.dyn.active = 0;
-      if (sh.plan.proto == kProtoFifo) sh.dyn.slice = 0;
-      sh.dyn.wait[0] = noWait();
-      sh.dyn.wait[1] = noWait();
       sh.taskq[qi] = (uint16_t)kInvalidTask;
-      sh.peersLoaded = 0;
-      // completion (manipulateCQ7ResetDoneColl, enqueue_ofccl_dev.cu:773-920): results are released to the
-      // system (unless the protocol has done so already), then the last channel to finish posts the entry
-      if (!sh.released) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-      bool last = true;
-      if (sh.plan.nChannels > 1) {
-        const uint64_t old = __hip_atomic_fetch_add(G(sh.plan.doneCounter), 1ull, __ATOMIC_ACQ_REL, DFCCL_AGENT);
-        last = ((old + 1) % (uint64_t)sh.plan.nChannels == 0);
-      }
-      if (last) {
-        // a rank with a single channel has a single poster, which keeps the ticket itself
-        const uint64_t t = (R.nChannels == 1) ? sh.cqNext++
-                                              : __hip_atomic_fetch_add(G(R.cqTicket), 1ull, __ATOMIC_RELAXED, DFCCL_AGENT);
-        const uint64_t cqe = cqeEncode((unsigned)ch, (unsigned)(t + 1), (unsigned)sh.plan.collId);
-        if (sh.released) __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]), cqe, __ATOMIC_RELAXED, DFCCL_SYSTEM);
-        else __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]), cqe, __ATOMIC_RELEASE, DFCCL_SYSTEM);
-        sh.stats.cqesWritten++;
-        trace(A, sh, kTrCqePosted, coll);
-      }
-      storeStruct(dynG, sh.dyn);
+      completeColl(A, R, sh, ch, coll);
     } else {
       // preempted: save the context (saveExcutingCollCtx, enqueue_ofccl_dev.cu:664-677)
       storeStruct(dynG, sh.dyn);
@@ -966,6 +1107,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     if (wave == 0) {
       if (ch == 0) pollHost(A, R, sh, lane);
       else ingestMirror(A, R, sh, ch, lane);
+      if (sh.ingested > 0 && sh.express) runExpress(A, R, sh, ch, lane);
       if (sh.numActive > 0) scanReady(R, sh, ch, lane);
       else if (lane == 0) sh.numReady = 0;
       if (lane == 0) {

@@ -119,6 +119,7 @@ struct alignas(16) CollPlan {
   PeerPub* pubs;           // [nRanks][nChannels]
   uint64_t* p1;            // [nRanks][nChannels] loops whose own chunk is folded and stored everywhere
   int64_t loopsPerInstance;
+  int64_t lastChunkElems;  // chunk size of the last loop (every other loop uses the nominal chunk)
 };
 
 // Resumable position of one collective on one workgroup (HBM). This is the
@@ -191,7 +192,8 @@ struct Knobs {
   int64_t tolerantUnprogressedCnt;  // TOLERANT_UNPROGRESSED_CNT, default 500000
   int64_t forceQuitEvery;           // DFCCL_FORCE_QUIT_EVERY: preempt after this many slices (0 = off)
   int64_t maxLifetimeTicks;         // DFCCL_DAEMON_MAX_MS in 100 MHz ticks (0 = unlimited)
-  int64_t idlePollRounds;           // DFCCL_IDLE_POLL_ROUNDS: x 4 pipelined polls per idle round of a leader (0 = off)
+  int64_t express;                  // DFCCL_EXPRESS: 0 switches the express path for small all-reduces off
+  int64_t idlePollRounds;           // DFCCL_IDLE_POLL_ROUNDS: 0 switches the pipelined polling of idle leaders off
 };
 
 struct DaemonArgs {

@@ -93,7 +93,7 @@ struct CommGroup {
   ConnFlags* flags = nullptr;
   // direct protocol
   int proto = kProtoFifo;
-  int64_t loopsPerInstance = 0;
+  int64_t loopsPerInstance = 0, lastChunkElems = 0;
   PeerPub* pubs = nullptr;   // [nRanks][nChannels]
   uint64_t* p1 = nullptr;    // [nRanks][nChannels]
 };
@@ -213,6 +213,7 @@ struct Daemon {
     knobs.tolerantUnprogressedCnt = envInt("TOLERANT_UNPROGRESSED_CNT", 500000);
     knobs.forceQuitEvery = envInt("DFCCL_FORCE_QUIT_EVERY", 0);
     knobs.maxLifetimeTicks = envInt("DFCCL_DAEMON_MAX_MS", 0) * 100000;  // wall_clock64 runs at 100 MHz
+    knobs.express = envInt("DFCCL_EXPRESS", 1);
     knobs.idlePollRounds = envInt("DFCCL_IDLE_POLL_ROUNDS", 8);
     if (knobs.numTryTaskqHead < 1) knobs.numTryTaskqHead = 1;
     if (knobs.tolerantUnprogressedCnt < 1) knobs.tolerantUnprogressedCnt = 1;
@@ -448,6 +449,9 @@ static void planGroup(CommGroup* g) {
   g->chanStride = g->slotBytes * g->fifoSlots;
   const int64_t loop = loopElems(g->kind, g->nRanks, g->nChannels, g->chunkElems);
   g->loopsPerInstance = g->count > 0 ? divUp64(g->count, loop) : 0;
+  g->lastChunkElems = g->count > 0 ? realChunkElems(g->kind, g->nRanks, g->nChannels, g->chunkElems, g->alignElems,
+                                                    g->count, (g->loopsPerInstance - 1) * loop)
+                                   : 0;
 }
 
 static ncclResult_t allocGroupLocked(CommGroup* g) {
@@ -784,6 +788,7 @@ DFCCL_API ncclResult_t ofcclFinalizeRankCtx7StartHostThrds(ofcclRankCtx_t c) {
     p.recvFifo = g->fifo ? g->fifo + (size_t)prev * g->nChannels * g->chanStride : nullptr;
     p.proto = g->proto; p.pad2 = 0; p.pubs = g->pubs; p.p1 = g->p1;
     p.loopsPerInstance = g->loopsPerInstance;
+    p.lastChunkElems = g->lastChunkElems;
     p.sendFlags = g->flags + (size_t)rank * g->nChannels;
     p.recvFlags = g->flags + (size_t)prev * g->nChannels;
     p.doneCounter = c->doneCounters + i;
