@@ -1208,3 +1208,7 @@ extern "C" hipError_t dfcclLaunchDaemon(const dfccl::DaemonArgs* devArgs, int nS
   return hipGetLastError();
 }
 
+// Workgroups of the daemon kernel one CU keeps resident.
+extern "C" hipError_t dfcclDaemonOccupancy(int* perCu) {
+  return hipOccupancyMaxActiveBlocksPerMultiprocessor(perCu, dfccl::dfcclDaemonKernel, dfccl::kWgThreads, 0);
+}

@@ -31,6 +31,7 @@
 
 #define DFCCL_API extern "C" __attribute__((visibility("default")))
 
+extern "C" hipError_t dfcclDaemonOccupancy(int* perCu);
 extern "C" hipError_t dfcclLaunchDaemon(const dfccl::DaemonArgs* devArgs, int nSlots, int channelsPerRank,
                                         hipStream_t stream);
 
@@ -183,10 +184,13 @@ struct Daemon {
   // workgroup that is not resident cannot answer its peers.
   long residentCapacity() {
     if (capacity > 0) return capacity;
-    // one 512-thread workgroup of the daemon kernel per CU (it needs more than 128 VGPRs per lane)
-    int cus = 0;
+    // every workgroup of the daemon has to be resident at the same time (they wait for each other): the grid
+    // may not exceed what the occupancy calculation says fits the GPU (one 512-thread workgroup per CU while
+    // the kernel needs more than 128 VGPRs per lane)
+    int cus = 0, perCu = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) cus = 0;
-    capacity = (long)cus;
+    if (dfcclDaemonOccupancy(&perCu) != hipSuccess || perCu < 1) perCu = 1;
+    capacity = (long)cus * perCu;
     return capacity;
   }
 
@@ -392,6 +396,9 @@ static void destroyDaemon(Daemon* d) {
 // Fixes the chunk geometry of the collective a communicator serves
 // (ofcclComputeColl / ofcclGetAlgoInfo, src/enqueue_ofccl.cc:85-283: ring, one
 // protocol, channel count shrunk for small messages).
+// Rank contexts alive per device: the workgroups of all of them have to fit the GPU together.
+static std::atomic<int> gLiveRankCtxs[64];
+
 static void planGroup(CommGroup* g) {
   const int es = typeSizeOf(g->dtypeUser);
   int64_t nBytes = (int64_t)g->countUser * es;
@@ -433,7 +440,11 @@ static void planGroup(CommGroup* g) {
     g->slicesPerChunk = 2;
     g->fifoSlots = 4;
   }
-  int maxCh = (int)envInt("NCCL_MAX_NCHANNELS", 32);
+  // Default: share the 256 workgroups that fill the GPU (one per CU) among the ranks that will run together,
+  // which is the larger of this communicator's size and the rank contexts created on the device so far.
+  int sharers = g->nRanks;
+  if (g->device >= 0 && g->device < 64) sharers = std::max(sharers, gLiveRankCtxs[g->device].load());
+  int maxCh = (int)envInt("NCCL_MAX_NCHANNELS", std::max(1, 256 / std::max(1, sharers)));
   if (maxCh < 1) maxCh = 1;
   if (maxCh > kMaxChannels) maxCh = kMaxChannels;
   const int64_t perChannel = envInt("DFCCL_BYTES_PER_CHANNEL", (int64_t)kWgThreads * 64);
@@ -725,6 +736,7 @@ DFCCL_API ncclResult_t ofcclInitRankCtx(ofcclRankCtx_t* rankCtx, int rank) {
     c->inflight[i].store(0);
     c->submitNs[i] = c->completeNs[i] = 0;
   }
+  if (device >= 0 && device < 64) gLiveRankCtxs[device].fetch_add(1);
   *rankCtx = c;
   return ncclSuccess;
 }
@@ -929,6 +941,7 @@ DFCCL_API ncclResult_t ofcclDestroy(ofcclRankCtx_t c) {
     }
   }
   for (auto& reg : c->colls) reg.comm->registered = false;
+  if (c->device >= 0 && c->device < 64) gLiveRankCtxs[c->device].fetch_sub(1);
   delete c;
   return ncclSuccess;
 }
