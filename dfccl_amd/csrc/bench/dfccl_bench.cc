@@ -384,6 +384,9 @@ static int runBuckets(const Args& a, bool single) {
   const double best = ms.empty() ? 0 : *std::min_element(ms.begin(), ms.end());
   const double med = pct(ms, 0.5);
   if (getenv("DFCCL_BENCH_VERBOSE")) {
+    fprintf(stderr, "iterations (ms):");
+    for (int it = (single ? 2 : 1); it < total; it++) fprintf(stderr, " %.3f", (double)(endNs[it].load() - tStart[it]) / 1e6);
+    fprintf(stderr, "\n");
     // last iteration, microseconds after rank 0's start stamp: last entry written, last completion seen by the
     // poller, waiting thread released
     for (int r = 0; r < n; r++)

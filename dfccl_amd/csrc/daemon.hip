@@ -35,6 +35,7 @@ namespace dfccl {
 
 constexpr int kDaemonUnroll = 1;  // see reduce_copy.hip: shallow unrolling keeps DRAM accesses ordered
 constexpr int kReadyWords = (kMaxColls + 63) / 64;
+constexpr int kSoftWaitSpins = 2;       // polls of a wait of the direct protocol while other collectives are queued
 constexpr int kExpressMaxBytes = 4096;  // largest own chunk wave 0 folds by itself (see runExpress)
 constexpr int kIdleRounds = 8;  // x 4 polls of the host ring before an idle leader goes round its main loop again
 enum RunStatus : int { kRunDone = 0, kRunPreempted = 1 };
@@ -205,6 +206,20 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
             sh.plan.lastChunkElems * sh.plan.elemSize <= kExpressMaxBytes && A.knobs.forceQuitEvery == 0 &&
             A.knobs.express != 0 && sh.dyn.step == 0)
           expressLane = true;
+      }
+    } else {
+      // Any other all-reduce of the direct protocol publishes its buffers here as well, straight from the
+      // context in HBM: its peers can then fold it whenever they get to it, whatever this workgroup is busy
+      // with, so that ranks which work through their collectives in different orders never wait for each
+      // other before the data has moved.
+      const DFCCL_GLOBAL CollPlan* pl = G(&R.plans[coll]);
+      if (pl->proto == kProtoDirect &&
+          __hip_atomic_load(G(&d->slice), __ATOMIC_RELAXED, DFCCL_AGENT) == 0) {
+        const uint64_t tag = pubTag(__hip_atomic_load(G(&d->instance), __ATOMIC_RELAXED, DFCCL_AGENT));
+        PeerPub* myPub = &pl->pubs[(size_t)pl->rank * pl->nChannels + ch];
+        __hip_atomic_store(G(&myPub->send), sendbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
+        __hip_atomic_store(G(&myPub->recv), recvbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
+        d->slice = 1;
       }
     }
     sh.taskq[base + pos] = (uint16_t)coll;
@@ -411,7 +426,7 @@ __device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, int ch
 // is bounded: when the budget is spent the collective is preempted.  (Role of
 // waitPeer, src/collectives_ofccl/device/ofccl_prims_simple.h:90-198.)  Returns the word the lane saw last.
 __device__ __forceinline__ uint64_t waitDescs(const DaemonArgs& A, WgShared& sh, int lane, const WaitDesc& w0,
-                                              const WaitDesc& w1, bool adapt) {
+                                              const WaitDesc& w1, bool adapt, int64_t cap = 0) {
   bool ok;
   int64_t spins = 0;
   uint64_t seen = 0;
@@ -429,7 +444,7 @@ __device__ __forceinline__ uint64_t waitDescs(const DaemonArgs& A, WgShared& sh,
       p = (const DFCCL_GLOBAL uint64_t*)(uintptr_t)(w.ptr + (uint64_t)((int64_t)idx * w.stride));
     const uint64_t need = w.value;
     bool ready = (p == nullptr);
-    const int64_t threshold = sh.threshold;
+    const int64_t threshold = (cap > 0 && cap < sh.threshold) ? cap : sh.threshold;
     for (;;) {
       if (!ready) {
         seen = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_AGENT);
@@ -445,7 +460,7 @@ __device__ __forceinline__ uint64_t waitDescs(const DaemonArgs& A, WgShared& sh,
     trace(A, sh, kTrWaitEnd, (uint32_t)((ok ? 1u : 0u) | ((uint32_t)spins << 1)));
     sh.waitOk = ok ? 1 : 0;
     sh.stats.spins += (uint64_t)spins;
-    if (ok && adapt) {
+    if (ok && adapt && cap == 0) {
       const int64_t t = A.knobs.recvSuccessFactor * spins;
       if (t > sh.threshold) sh.threshold = t;
     }
@@ -739,6 +754,9 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
   PeerPub* myPub = &P.pubs[(size_t)me * C + ch];
   const int64_t l0 = sh.dyn.gridOffset;
   const int phase = sh.dyn.step;
+  // With other collectives queued a wait is only a look: switching is cheap here (contexts are small and
+  // nothing is held while parked), and the workgroup is better off moving the next collective's data.
+  const int64_t cap = (sh.numActive > 1 && forceEvery == 0) ? kSoftWaitSpins : 0;
   __syncthreads();  // every thread has taken its copy of the position before thread 0 changes it
 
   if (!published && tid < 2) {
@@ -756,7 +774,7 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
       const WaitDesc w0 = waitFor(&P.pubs[ch].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
       const WaitDesc w1 = waitFor(&P.pubs[ch].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
       if (wave == 0) {
-        const uint64_t word = waitDescs(A, sh, lane, w0, w1, true);
+        const uint64_t word = waitDescs(A, sh, lane, w0, w1, true, cap);
         if (sh.waitOk && (lane & 31) < n) {
           // sources in fold order, destinations by rank
           if (lane < 32) sh.sweep.src[(lane + n - 1 - me) % n] = word & kPtrMask;
@@ -835,7 +853,7 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
   if (phase != 0 && tid == 0) sh.released = 1;  // resumed here: the sweep's release was done before it was parked
   {
     const WaitDesc w0 = waitFor(&P.p1[ch], base + (uint64_t)L, ctrStride, n);
-    if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true);
+    if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true, cap);
     __syncthreads();
     if (!sh.waitOk) {
       if (tid == 0) {

@@ -522,7 +522,7 @@ static ncclResult_t prepareColl(int kind, size_t count, int dtype, int op, int r
 // Consumes the completion ring in ticket order and fires the callbacks
 // (startPoller / cqRead, src/enqueue_ofccl.cc:908-965,697-739).
 static void pollerLoop(ofcclRankCtx* c) {
-  uint64_t emptySpins = 0;
+  uint64_t emptySpins = 0, waitingSince = 0;
   while (!c->stopPoller.load(std::memory_order_acquire)) {
     const uint64_t v = __atomic_load_n(&c->dev.cq[c->cqRead & (kCqRing - 1)], __ATOMIC_ACQUIRE);
     if (v != ~0ull && cqeCnt(v) == (unsigned)((c->cqRead + 1) & 0xffffffu)) {
@@ -530,6 +530,7 @@ static void pollerLoop(ofcclRankCtx* c) {
       const int collId = (int)cqeCollId(v);
       c->cqRead++;
       emptySpins = 0;
+      waitingSince = 0;
       if (collId >= 0 && collId < kMaxColls) {
         CallbackFunc cb = c->callbacks[collId];
         void* args = c->cbArgs[collId];
@@ -550,8 +551,13 @@ static void pollerLoop(ofcclRankCtx* c) {
       });
       c->pollerAsleep.store(false);
       emptySpins = 0;
-    } else if (++emptySpins > 20000) {
-      sched_yield();
+      waitingSince = 0;
+    } else if ((++emptySpins & 1023u) == 0) {
+      // work is outstanding: keep spinning (giving the CPU away here costs a scheduler slice when it is least
+      // affordable); only a completion that has not come for milliseconds is waited for at a lower rate
+      const uint64_t now = nowNs();
+      if (waitingSince == 0) waitingSince = now;
+      else if (now - waitingSince > 5000000ull) usleep(50);
     } else {
       _mm_pause();
     }
