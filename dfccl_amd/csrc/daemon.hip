@@ -44,6 +44,9 @@ enum RunStatus : int { kRunDone = 0, kRunPreempted = 1 };
 // nChannels * n chunks of `real` elements; every loop but the last uses the nominal chunk.
 struct SweepGeom {
   int64_t count, loop, chunkElems, lastReal, L;
+  int64_t T;                         // tiles (one rank's chunk of one channel slot of one loop) per rank: L * C
+  uint64_t instBase;                 // value of the rank's tile counter when this instance began
+  uint64_t ctr;                      // the rank's tile counter
   int n, C, ch, es;
   int me, dtype, op, pad;
   uint64_t src[kMaxDirectRanks];     // the send buffers in fold order: in[me + 1], in[me + 2], ..., in[me]
@@ -82,6 +85,7 @@ struct WgShared {
   DynCtx dyn;
   WgStats stats;
   SweepGeom sweep;         // arguments of the direct protocol's sweeps
+  uint64_t ticket[2];      // tile numbers handed from thread 0 to the workgroup (two slots, used alternately)
   uint64_t ready[kReadyWords];
   uint16_t taskq[kMaxColls];
   uint8_t collChannels[kMaxColls];  // channels of every collective of this rank (copied from the plans at launch)
@@ -580,38 +584,91 @@ __device__ __forceinline__ int64_t sweepReal(const SweepGeom& g, int64_t l) {
   return (l == g.L - 1) ? g.lastReal : g.chunkElems;
 }
 
-// The sweep of the direct all-reduce: for loops [lBegin, lEnd) fold my own chunk from all n send buffers and
-// write the result into all n receive buffers.  All workgroups sweep the loops together, so at any instant the
-// accesses of the whole grid fall into one window of nChannels * n chunks per buffer.
+// The sweep of the direct all-reduce.  A tile is my rank's chunk in one channel slot of one loop: tile t lies in
+// loop t / C, slot t % C, at l * loop + (slot * n + me) * real.  For every tile it takes, the workgroup folds the
+// chunk from all n send buffers and writes the result into all n receive buffers.  Tiles are handed out low to
+// high, so at any instant the accesses of the whole grid fall into a narrow window of every buffer.
+//  * With one channel the workgroup takes the tiles in order; `pos` is the next tile.
+//  * With several channels the first loop is static (workgroup ch takes tile ch; pos 0 = not done yet) and the
+//    rest is handed out by the rank's tile counter, whichever workgroup is free next: workgroups do not finish
+//    at the same moment otherwise (HBM channels are not equally fast for all of them), and the slowest one
+//    decides when the collective is done.  The next tile is requested while the current one is folded.  Every
+//    workgroup draws exactly one number past the end per instance, so the counter advances by exactly T.
+// At most maxTiles tiles are processed; `finished` says that no tile is left.
 template <int DT, int OP, int NS>
-__device__ __forceinline__ void sweepFoldN(const SweepGeom& g, int64_t lBegin, int64_t lEnd, int tid) {
-  for (int64_t l = lBegin; l < lEnd; l++) {
-    const int64_t real = sweepReal(g, l);
-    const int64_t off = l * g.loop + ((int64_t)g.ch * g.n + g.me) * real;
+__device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, int64_t& posInOut, int64_t maxTiles,
+                                           int tid, int64_t& tilesDone, bool& finished) {
+  const bool dynamic = g.C > 1;
+  DFCCL_GLOBAL uint64_t* ctr = (DFCCL_GLOBAL uint64_t*)(uintptr_t)g.ctr;
+  int64_t pos = posInOut, done = 0;
+  bool fin = false, have = false;
+  uint64_t tile = 0;
+  uint32_t par = 0;
+  while (done < maxTiles) {
+    if (!have) {
+      if (!dynamic) {
+        tile = (uint64_t)pos++;
+      } else if (pos == 0) {
+        tile = (uint64_t)g.ch;
+        pos = 1;
+      } else {
+        if (tid == 0)
+          slots[par] = __hip_atomic_fetch_add(ctr, 1ull, __ATOMIC_RELAXED, DFCCL_AGENT) - g.instBase + (uint64_t)g.C;
+        __syncthreads();
+        tile = slots[par];
+        par ^= 1u;
+      }
+    }
+    have = false;
+    if (tile >= (uint64_t)g.T) {
+      fin = true;
+      break;
+    }
+    const bool prefetch = dynamic && done + 1 < maxTiles;
+    uint64_t nxt = 0;
+    if (prefetch && tid == 0)
+      nxt = __hip_atomic_fetch_add(ctr, 1ull, __ATOMIC_RELAXED, DFCCL_AGENT) - g.instBase + (uint64_t)g.C;
+    const uint32_t l = (uint32_t)tile / (uint32_t)g.C, slot = (uint32_t)tile % (uint32_t)g.C;
+    const int64_t real = ((int64_t)l == g.L - 1) ? g.lastReal : g.chunkElems;
+    const int64_t off = (int64_t)l * g.loop + ((int64_t)slot * g.n + g.me) * real;
     const int64_t nelem = (g.count - off < real) ? g.count - off : real;
     if (nelem > 0) foldTile<DT, OP, NS>(g.src, g.dst, g.n, off * g.es, (size_t)(nelem * g.es), tid);
+    done++;
+    if (prefetch) {
+      if (tid == 0) slots[par] = nxt;
+      __syncthreads();
+      tile = slots[par];
+      par ^= 1u;
+      have = true;
+    }
   }
+  posInOut = pos;
+  tilesDone = done;
+  finished = fin;
 }
 
 template <int DT, int OP>
-__device__ __forceinline__ void sweepFold(const SweepGeom& g, int64_t lBegin, int64_t lEnd, int tid) {
-  if (g.n <= 2) sweepFoldN<DT, OP, 2>(g, lBegin, lEnd, tid);
-  else if (g.n <= 4) sweepFoldN<DT, OP, 4>(g, lBegin, lEnd, tid);
-  else sweepFoldN<DT, OP, 8>(g, lBegin, lEnd, tid);
+__device__ __forceinline__ void sweepFold(const SweepGeom& g, uint64_t* slots, int64_t& pos, int64_t maxTiles, int tid,
+                                          int64_t& tilesDone, bool& finished) {
+  if (g.n <= 2) sweepFoldN<DT, OP, 2>(g, slots, pos, maxTiles, tid, tilesDone, finished);
+  else if (g.n <= 4) sweepFoldN<DT, OP, 4>(g, slots, pos, maxTiles, tid, tilesDone, finished);
+  else sweepFoldN<DT, OP, 8>(g, slots, pos, maxTiles, tid, tilesDone, finished);
 }
 
 template <int DT>
-__device__ __forceinline__ void sweepFoldOp(int op, const SweepGeom& g, int64_t lBegin, int64_t lEnd, int tid) {
+__device__ __forceinline__ void sweepFoldOp(int op, const SweepGeom& g, uint64_t* slots, int64_t& pos, int64_t maxTiles,
+                                            int tid, int64_t& tilesDone, bool& finished) {
   switch (op) {
-    case kSum: sweepFold<DT, kSum>(g, lBegin, lEnd, tid); break;
-    case kProd: sweepFold<DT, kProd>(g, lBegin, lEnd, tid); break;
-    case kMax: sweepFold<DT, kMax>(g, lBegin, lEnd, tid); break;
-    default: sweepFold<DT, kMin>(g, lBegin, lEnd, tid); break;
+    case kSum: sweepFold<DT, kSum>(g, slots, pos, maxTiles, tid, tilesDone, finished); break;
+    case kProd: sweepFold<DT, kProd>(g, slots, pos, maxTiles, tid, tilesDone, finished); break;
+    case kMax: sweepFold<DT, kMax>(g, slots, pos, maxTiles, tid, tilesDone, finished); break;
+    default: sweepFold<DT, kMin>(g, slots, pos, maxTiles, tid, tilesDone, finished); break;
   }
 }
 
 // The geometry and the buffer tables are handed over in LDS and copied to registers here.
-__device__ __forceinline__ void sweepFoldAny(const SweepGeom* gp, int64_t lBegin, int64_t lEnd, int tid) {
+__device__ __forceinline__ void sweepFoldAny(const SweepGeom* gp, uint64_t* slots, int64_t& pos, int64_t maxTiles,
+                                             int tid, int64_t& tilesDone, bool& finished) {
   SweepGeom g = *gp;
 #pragma unroll
   for (int t = 0; t < kMaxDirectRanks; t++) {
@@ -620,11 +677,11 @@ __device__ __forceinline__ void sweepFoldAny(const SweepGeom* gp, int64_t lBegin
   }
   const int op = g.op;
   switch (g.dtype) {
-    case kF32: sweepFoldOp<kF32>(op, g, lBegin, lEnd, tid); break;
-    case kBF16: sweepFoldOp<kBF16>(op, g, lBegin, lEnd, tid); break;
-    case kF16: sweepFoldOp<kF16>(op, g, lBegin, lEnd, tid); break;
-    case kI32: sweepFoldOp<kI32>(op, g, lBegin, lEnd, tid); break;
-    default: sweepFoldOp<kI8>(op, g, lBegin, lEnd, tid); break;
+    case kF32: sweepFoldOp<kF32>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
+    case kBF16: sweepFoldOp<kBF16>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
+    case kF16: sweepFoldOp<kF16>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
+    case kI32: sweepFoldOp<kI32>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
+    default: sweepFoldOp<kI8>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
   }
 }
 
@@ -791,6 +848,9 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
           g.chunkElems = P.chunkElems;
           g.lastReal = P.lastChunkElems;
           g.L = L;
+          g.T = L * C;
+          g.instBase = inst * (uint64_t)(L * C);
+          g.ctr = (uint64_t)(uintptr_t)P.tileCtr;
           g.n = n;
           g.C = C;
           g.ch = ch;
@@ -807,15 +867,17 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
     }
 
     if (tid == 0) trace(A, sh, kTrMoveBegin, 0);
+    int64_t pos = l0, tilesDone = 0;
+    bool finished = false;
     if (forceEvery > 0) {
-      // test hook: one loop at a time, with a preemption point before each
-      for (int64_t l = l0; l < L; l++) {
+      // test hook: one tile at a time, with a preemption point before each
+      while (!finished) {
         __syncthreads();
         if (sh.slicesSinceLoad >= forceEvery) {
           __syncthreads();
           if (tid == 0) {
             sh.stats.forcedQuits++;
-            sh.dyn.gridOffset = l;
+            sh.dyn.gridOffset = pos;
             sh.dyn.step = 0;
             sh.dyn.wait[0] = noWait();
             sh.dyn.wait[1] = noWait();
@@ -823,19 +885,19 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
           return kRunPreempted;
         }
         __syncthreads();
-        sweepFoldAny(&sh.sweep, l, l + 1, tid);
-        if (tid == 0) {
+        sweepFoldAny(&sh.sweep, sh.ticket, pos, 1, tid, tilesDone, finished);
+        if (tid == 0 && tilesDone > 0) {
           sh.progressed = 1;
-          sh.slicesSinceLoad++;
-          sh.stats.slicesMoved++;
+          sh.slicesSinceLoad += tilesDone;
+          sh.stats.slicesMoved += (uint64_t)tilesDone;
         }
       }
     } else {
-      sweepFoldAny(&sh.sweep, l0, L, tid);
+      sweepFoldAny(&sh.sweep, sh.ticket, pos, INT64_MAX, tid, tilesDone, finished);
       if (tid == 0) {
         sh.progressed = 1;
-        sh.slicesSinceLoad += L - l0;
-        sh.stats.slicesMoved += (uint64_t)(L - l0);
+        sh.slicesSinceLoad += tilesDone;
+        sh.stats.slicesMoved += (uint64_t)tilesDone;
       }
     }
     __syncthreads();

@@ -120,6 +120,7 @@ struct alignas(16) CollPlan {
   uint64_t* p1;            // [nRanks][nChannels] loops whose own chunk is folded and stored everywhere
   int64_t loopsPerInstance;
   int64_t lastChunkElems;  // chunk size of the last loop (every other loop uses the nominal chunk)
+  uint64_t* tileCtr;       // direct protocol, several channels: this rank's tile counter (see sweepFoldN)
 };
 
 // Resumable position of one collective on one workgroup (HBM). This is the

@@ -15,6 +15,8 @@ namespace dfccl {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef short i16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 // Values of ncclDataType_t / ncclRedOp_t that this path implements.
 enum : int { kI8 = 0, kI32 = 2, kF16 = 6, kF32 = 7, kBF16 = 9 };
@@ -30,13 +32,6 @@ __device__ __forceinline__ float opF32(float a, float b) {
   else if constexpr (OP == kProd) return a * b;
   else if constexpr (OP == kMax) return __builtin_fmaxf(a, b);
   else return __builtin_fminf(a, b);
-}
-
-// float -> bfloat16 bits, round to nearest even (NaN inputs are outside the
-// supported domain of the parity tests).
-__device__ __forceinline__ uint32_t bf16Round(float f) {
-  uint32_t u = __float_as_uint(f);
-  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
 }
 
 template <int DT, int OP>
@@ -56,9 +51,13 @@ __device__ __forceinline__ uint32_t wordOp(uint32_t a, uint32_t b) {
     else r = __builtin_elementwise_min(x, y);
     return __builtin_bit_cast(uint32_t, r);
   } else if constexpr (DT == kBF16) {
+    // widen (exact), operate in fp32, round both results to bfloat16 (nearest even) with one v_cvt_pk_bf16_f32
     float alo = __uint_as_float(a << 16), ahi = __uint_as_float(a & 0xffff0000u);
     float blo = __uint_as_float(b << 16), bhi = __uint_as_float(b & 0xffff0000u);
-    return bf16Round(opF32<OP>(alo, blo)) | (bf16Round(opF32<OP>(ahi, bhi)) << 16);
+    f32x2 r;
+    r.x = opF32<OP>(alo, blo);
+    r.y = opF32<OP>(ahi, bhi);
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(r, bf16x2));
   } else {  // int8, four per word
     if constexpr (OP == kSum) {
       // add even and odd bytes separately so that carries cannot cross a byte

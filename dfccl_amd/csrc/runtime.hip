@@ -96,7 +96,8 @@ struct CommGroup {
   int proto = kProtoFifo;
   int64_t loopsPerInstance = 0, lastChunkElems = 0;
   PeerPub* pubs = nullptr;   // [nRanks][nChannels]
-  uint64_t* p1 = nullptr;    // [nRanks][nChannels]
+  uint64_t* p1 = nullptr;        // [nRanks][nChannels]
+  uint64_t* tileCtrs = nullptr;  // [nRanks] x 128 bytes
 };
 
 }  // namespace dfccl
@@ -477,6 +478,8 @@ static ncclResult_t allocGroupLocked(CommGroup* g) {
     HIPCHECK(hipMemset(g->pubs, 0, links * sizeof(PeerPub)));
     HIPCHECK(hipMalloc((void**)&g->p1, links * 8));
     HIPCHECK(hipMemset(g->p1, 0, links * 8));
+    HIPCHECK(hipMalloc((void**)&g->tileCtrs, (size_t)g->nRanks * 128));
+    HIPCHECK(hipMemset(g->tileCtrs, 0, (size_t)g->nRanks * 128));
   }
   return ncclSuccess;
 }
@@ -690,12 +693,12 @@ DFCCL_API ncclResult_t ncclCommDestroy(ncclComm_t comm) {
     if (d != nullptr) {
       std::lock_guard<std::mutex> lk(d->mu);
       if (d->running) {
-        for (void* p : {(void*)g->fifo, (void*)g->flags, (void*)g->pubs, (void*)g->p1})
+        for (void* p : {(void*)g->fifo, (void*)g->flags, (void*)g->pubs, (void*)g->p1, (void*)g->tileCtrs})
           if (p) d->garbageDev.push_back(p);
-        g->fifo = nullptr; g->flags = nullptr; g->pubs = nullptr; g->p1 = nullptr;
+        g->fifo = nullptr; g->flags = nullptr; g->pubs = nullptr; g->p1 = nullptr; g->tileCtrs = nullptr;
       }
     }
-    for (void* p : {(void*)g->fifo, (void*)g->flags, (void*)g->pubs, (void*)g->p1})
+    for (void* p : {(void*)g->fifo, (void*)g->flags, (void*)g->pubs, (void*)g->p1, (void*)g->tileCtrs})
       if (p) (void)hipFree(p);
     delete g;
   }
@@ -807,6 +810,7 @@ DFCCL_API ncclResult_t ofcclFinalizeRankCtx7StartHostThrds(ofcclRankCtx_t c) {
     p.proto = g->proto; p.pad2 = 0; p.pubs = g->pubs; p.p1 = g->p1;
     p.loopsPerInstance = g->loopsPerInstance;
     p.lastChunkElems = g->lastChunkElems;
+    p.tileCtr = g->tileCtrs ? g->tileCtrs + (size_t)rank * 16 : nullptr;
     p.sendFlags = g->flags + (size_t)rank * g->nChannels;
     p.recvFlags = g->flags + (size_t)prev * g->nChannels;
     p.doneCounter = c->doneCounters + i;
