@@ -108,7 +108,7 @@ def run_native(args, env=None, timeout=180):
 
 def bench_daemon_all_reduce():
     """Ring all-reduce over 8 virtual ranks, bf16 Sum, 64 MiB per rank, through the daemon kernel: once with
-    the library's defaults (direct protocol, 16 KiB interleave grain) and once as the FIFO ring with 512 KiB
+    the library's defaults (direct protocol, 8 KiB tiles) and once as the FIFO ring with 512 KiB
     chunks. GB/s figures are on the bytes the respective schedule moves."""
     n, nbytes = 8, 64 << 20
     res = {}

@@ -954,7 +954,11 @@ __device__ __forceinline__ void completeColl(const DaemonArgs& A, const RankDev&
   if (!sh.released) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
   bool last = true;
   if (sh.plan.nChannels > 1) {
-    const uint64_t old = __hip_atomic_fetch_add(G(sh.plan.doneCounter), 1ull, __ATOMIC_ACQ_REL, DFCCL_AGENT);
+    // (with the results released already there is nothing left to write back: acquire is enough, and spares
+    // the completion a walk through the L2)
+    const uint64_t old = sh.released
+                             ? __hip_atomic_fetch_add(G(sh.plan.doneCounter), 1ull, __ATOMIC_ACQUIRE, DFCCL_AGENT)
+                             : __hip_atomic_fetch_add(G(sh.plan.doneCounter), 1ull, __ATOMIC_ACQ_REL, DFCCL_AGENT);
     last = ((old + 1) % (uint64_t)sh.plan.nChannels == 0);
   }
   if (last) {

@@ -426,7 +426,7 @@ static void planGroup(CommGroup* g) {
   if (g->proto == kProtoDirect) {
     // no FIFO: the chunk is only the interleaving grain of the sweeps (small grains keep all workgroups
     // inside one compact address window per buffer)
-    chunkBytes = roundUp64(std::max<int64_t>(envInt("DFCCL_DIRECT_CHUNK_BYTES", 16 << 10), kAlignBytes), kAlignBytes);
+    chunkBytes = roundUp64(std::max<int64_t>(envInt("DFCCL_DIRECT_CHUNK_BYTES", 8 << 10), kAlignBytes), kAlignBytes);
     sliceBytes = chunkBytes;
     g->slicesPerChunk = 1;
     g->fifoSlots = 1;

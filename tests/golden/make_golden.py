@@ -18,18 +18,18 @@ import datagen  # noqa: E402
 import dfccl_oracle as orc  # noqa: E402
 
 # kind, dtype, op, n, count, root, (nChannels, chunkElems, alignElems)
-# The float all-reduce cases use the geometry the library plans for these sizes (one channel, 16 KiB chunks,
+# The float all-reduce cases use the geometry the library plans for these sizes (one channel, 8 KiB chunks,
 # 1 KiB rounding), so that the GPU suite can compare them bit for bit.
 CASES = [
-    ("all_reduce", orc.F32, orc.SUM, 2, 1000, 0, (1, 4096, 256)),
-    ("all_reduce", orc.F32, orc.SUM, 4, 2048, 0, (1, 4096, 256)),
-    ("all_reduce", orc.BF16, orc.SUM, 8, 4100, 0, (1, 8192, 512)),
-    ("all_reduce", orc.F16, orc.SUM, 4, 2048, 0, (1, 8192, 512)),
-    ("all_reduce", orc.F16, orc.PROD, 3, 777, 0, (1, 8192, 512)),
+    ("all_reduce", orc.F32, orc.SUM, 2, 1000, 0, (1, 2048, 256)),
+    ("all_reduce", orc.F32, orc.SUM, 4, 2048, 0, (1, 2048, 256)),
+    ("all_reduce", orc.BF16, orc.SUM, 8, 4100, 0, (1, 4096, 512)),
+    ("all_reduce", orc.F16, orc.SUM, 4, 2048, 0, (1, 4096, 512)),
+    ("all_reduce", orc.F16, orc.PROD, 3, 777, 0, (1, 4096, 512)),
     ("all_reduce", orc.I32, orc.SUM, 5, 1234, 0, (2, 256, 256)),
     ("all_reduce", orc.I8, orc.MIN, 4, 5000, 0, (1, 1024, 1024)),
     ("all_reduce", orc.F32, orc.MAX, 8, 900, 0, (1, 256, 256)),
-    ("all_reduce", orc.BF16, orc.PROD, 2, 513, 0, (1, 8192, 512)),
+    ("all_reduce", orc.BF16, orc.PROD, 2, 513, 0, (1, 4096, 512)),
     ("reduce_scatter", orc.F32, orc.SUM, 4, 700, 0, (1, 256, 256)),
     ("reduce_scatter", orc.BF16, orc.SUM, 3, 1025, 0, (2, 512, 512)),
     ("reduce_scatter", orc.I8, orc.MAX, 8, 300, 0, (1, 1024, 1024)),
