@@ -47,8 +47,9 @@ struct SweepGeom {
   int64_t T;                         // tiles (one rank's chunk of one channel slot of one loop) per rank: L * C
   uint64_t instBase;                 // value of the rank's tile counter when this instance began
   uint64_t ctr;                      // the rank's tile counter
-  int n, C, ch, es;
-  int me, dtype, op, pad;
+  int n, C, ch, es;                  // n: sources folded (1 = plain copy)
+  int me, dtype, op, nd;             // nd: destinations written
+  int tn, tme, pad0, pad1;           // a loop holds C * tn chunks, mine is number tme of every channel slot
   uint64_t src[kMaxDirectRanks];     // the send buffers in fold order: in[me + 1], in[me + 2], ..., in[me]
   uint64_t dst[kMaxDirectRanks];     // every rank's receive buffer
 };
@@ -84,6 +85,8 @@ struct WgShared {
   CollPlan plan;
   DynCtx dyn;
   WgStats stats;
+  uint64_t peerSend[kMaxDirectRanks];  // direct protocol: the buffers the ranks have published
+  uint64_t peerRecv[kMaxDirectRanks];
   SweepGeom sweep;         // arguments of the direct protocol's sweeps
   uint64_t ticket[2];      // tile numbers handed from thread 0 to the workgroup (two slots, used alternately)
   uint64_t ready[kReadyWords];
@@ -206,7 +209,8 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
         __hip_atomic_store(G(&myPub->recv), recvbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
         sh.dyn.slice = 1;
         // alone in the queue and small: wave 0 can run it on the spot (see runExpress)
-        if (base == 0 && __builtin_popcountll(mm) == 1 && sh.plan.nChannels == 1 && sh.plan.loopsPerInstance == 1 &&
+        if (base == 0 && __builtin_popcountll(mm) == 1 && sh.plan.kind == kAllReduce && sh.plan.nChannels == 1 &&
+            sh.plan.loopsPerInstance == 1 &&
             sh.plan.lastChunkElems * sh.plan.elemSize <= kExpressMaxBytes && A.knobs.forceQuitEvery == 0 &&
             A.knobs.express != 0 && sh.dyn.step == 0)
           expressLane = true;
@@ -536,19 +540,21 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
   return (uint64_t)lo | ((uint64_t)hi << 32);
 }
 
-// dst[k][off..] = src[0][off..] (op) src[1][off..] ... (op) src[n-1][off..] for every k < n, folded left to
+// dst[k][off..] = src[0][off..] (op) src[1][off..] ... (op) src[n-1][off..] for every k < nd, folded left to
 // right with every step rounded to the storage type: with src = in[c+1], in[c+2], ..., in[c] this is the ring's
-// order for a chunk owned by rank c.  n <= NS <= kMaxDirectRanks; the NS - n surplus loads re-read src[0] (they
-// hit in cache) so that every array element is defined: predicated loads made the compiler keep the packs in
-// scratch.  A destination may be one of the sources (in place): each thread reads a pack before it writes it,
-// and no other thread touches that pack.
+// order for a chunk owned by rank c.  n <= NS <= kMaxDirectRanks (NS = 1: plain copy); the NS - n surplus loads
+// re-read src[0] (they hit in cache) so that every array element is defined: predicated loads made the compiler
+// keep the packs in scratch.  A destination may be one of the sources (in place): each thread reads a pack
+// before it writes it, and no other thread touches that pack.
 template <int DT, int OP, int NS>
 __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks], const uint64_t (&dst)[kMaxDirectRanks],
-                                         int n, int64_t byteOff, size_t nbytes, int tid) {
+                                         int n, int nd, int64_t byteOff, size_t nbytes, int tid) {
   constexpr int ES = typeSize(DT);
   uint64_t align = (uint64_t)byteOff;
 #pragma unroll
-  for (int j = 0; j < NS; j++) align |= src[j] | (j < n ? dst[j] : 0);
+  for (int j = 0; j < NS; j++) align |= (j < n ? src[j] : 0);
+#pragma unroll
+  for (int j = 0; j < kMaxDirectRanks; j++) align |= (j < nd ? dst[j] : 0);
   size_t doneBytes = 0;
   if ((align & 15u) == 0) {
     const size_t npacks = nbytes >> 4;
@@ -562,8 +568,8 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
       for (int j = 1; j < NS; j++)
         if (j < n) acc = packOp<DT, OP>(acc, v[j]);
 #pragma unroll
-      for (int j = 0; j < NS; j++)
-        if (j < n) storePack<false>((char*)dst[j] + byteOff, i, acc);
+      for (int j = 0; j < kMaxDirectRanks; j++)
+        if (j < nd) storePack<false>((char*)dst[j] + byteOff, i, acc);
     }
     doneBytes = npacks << 4;
   }
@@ -575,18 +581,15 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
     for (int j = 1; j < NS; j++)
       if (j < n) acc = wordOp<DT, OP>(acc, loadElem<ES>((const char*)src[j] + byteOff, i));
 #pragma unroll
-    for (int j = 0; j < NS; j++)
-      if (j < n) storeElem<ES>((char*)dst[j] + byteOff, i, acc);
+    for (int j = 0; j < kMaxDirectRanks; j++)
+      if (j < nd) storeElem<ES>((char*)dst[j] + byteOff, i, acc);
   }
 }
 
-__device__ __forceinline__ int64_t sweepReal(const SweepGeom& g, int64_t l) {
-  return (l == g.L - 1) ? g.lastReal : g.chunkElems;
-}
-
-// The sweep of the direct all-reduce.  A tile is my rank's chunk in one channel slot of one loop: tile t lies in
-// loop t / C, slot t % C, at l * loop + (slot * n + me) * real.  For every tile it takes, the workgroup folds the
-// chunk from all n send buffers and writes the result into all n receive buffers.  Tiles are handed out low to
+// The sweep of the direct protocol.  A tile is my rank's chunk in one channel slot of one loop: tile t lies in
+// loop t / C, slot t % C, at l * loop + (slot * tn + tme) * real (tn = ranks that share the index space, tme = my
+// place among them).  For every tile it takes, the workgroup folds the chunk from the n sources and writes the
+// result into the nd destinations.  Tiles are handed out low to
 // high, so at any instant the accesses of the whole grid fall into a narrow window of every buffer.
 //  * With one channel the workgroup takes the tiles in order; `pos` is the next tile.
 //  * With several channels the first loop is static (workgroup ch takes tile ch; pos 0 = not done yet) and the
@@ -630,9 +633,9 @@ __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, 
       nxt = __hip_atomic_fetch_add(ctr, 1ull, __ATOMIC_RELAXED, DFCCL_AGENT) - g.instBase + (uint64_t)g.C;
     const uint32_t l = (uint32_t)tile / (uint32_t)g.C, slot = (uint32_t)tile % (uint32_t)g.C;
     const int64_t real = ((int64_t)l == g.L - 1) ? g.lastReal : g.chunkElems;
-    const int64_t off = (int64_t)l * g.loop + ((int64_t)slot * g.n + g.me) * real;
+    const int64_t off = (int64_t)l * g.loop + ((int64_t)slot * g.tn + g.tme) * real;
     const int64_t nelem = (g.count - off < real) ? g.count - off : real;
-    if (nelem > 0) foldTile<DT, OP, NS>(g.src, g.dst, g.n, off * g.es, (size_t)(nelem * g.es), tid);
+    if (nelem > 0) foldTile<DT, OP, NS>(g.src, g.dst, g.n, g.nd, off * g.es, (size_t)(nelem * g.es), tid);
     done++;
     if (prefetch) {
       if (tid == 0) slots[par] = nxt;
@@ -676,6 +679,10 @@ __device__ __forceinline__ void sweepFoldAny(const SweepGeom* gp, uint64_t* slot
     g.dst[t] = uniform64(g.dst[t]);
   }
   const int op = g.op;
+  if (g.n <= 1) {  // plain copy, whatever the type
+    sweepFoldN<kI8, kSum, 1>(g, slots, pos, maxTiles, tid, tilesDone, finished);
+    return;
+  }
   switch (g.dtype) {
     case kF32: sweepFoldOp<kF32>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
     case kBF16: sweepFoldOp<kBF16>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
@@ -777,25 +784,32 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
 
 // ----------------------------------------------------------------- direct protocol
 
-// All-reduce in which the virtual ranks, whose buffers share one HBM, read each
+// Collectives in which the virtual ranks, whose buffers share one HBM, read each
 // other's send buffers and write each other's receive buffers in place.
-// Chunks are laid out as in the FIFO ring (ring_schedule.h): loop l, channel c,
-// chunk j (owned by rank j) starts at l * loop + (c * n + j) * real.
-//   publish   my buffers for this instance; wait until every peer has published
-//             (its receive buffer may be written from then on);
-//   sweep     all loops: fold my own chunk from the n send buffers, in the ring's
-//             order for that chunk, and store the result into all n receive
-//             buffers; release; p1[me] = loops done;
-//   finally   wait until every peer's p1 covers the instance: every chunk of my
-//             receive buffer has been written and nobody reads my send buffer any
+//   publish   my buffers for this instance (normally done when the submission was
+//             ingested); wait until every peer has published (its receive buffer
+//             may be written from then on);
+//   sweep     my share of the work, tile by tile: fold the sources in the ring's
+//             order for those elements and store the result into the destinations;
+//             release; p1[me] = loops done;
+//   finally   wait until every peer's p1 covers the instance: everything that had
+//             to land in my receive buffer has, and nobody reads my send buffer any
 //             more, so the completion may be posted.
-// Every input element is read once and every output element written once: 2N of
-// traffic per rank for a message of N bytes, against (6n-4)/n * N of the FIFO ring.
+// What "my share", sources and destinations are (n ranks, me, root; chunks as in
+// ring_schedule.h: loop l, channel slot c, chunk j starts at l * loop + (c * n + j) * real):
+//   all-reduce      the chunks owned by me;  in[me+1], ..., in[me] (the order in which the ring
+//                   accumulates a chunk that ends at its owner)  ->  every receive buffer
+//   reduce          the chunks owned by me;  in[root+1], ..., in[root]  ->  the root's receive buffer
+//   broadcast       the chunks owned by me;  the root's send buffer  ->  every receive buffer
+//   reduce-scatter  all of block me of the send buffers;  in[me+1], ..., in[me]  ->  my receive buffer
+//   all-gather      all of my send buffer  ->  block me of every receive buffer
+// Every input element is read once and every output element written once, against
+// the FIFO ring's staging of every slice through HBM at every step.
 // Two waits per instance whatever its size; each is a WaitDesc and can preempt.
 // dyn.step is the phase (0 = sweep, 2 = only the final wait is left),
-// dyn.gridOffset the next loop of the sweep, dyn.slice whether the instance is
-// published.
-__device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
+// dyn.gridOffset the sweep's position (see sweepFoldN), dyn.slice whether the
+// instance is published.
+__device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
   const CollPlan& P = sh.plan;
   const int lane = tid & 63, wave = tid >> 6;
   const int n = P.nRanks, C = P.nChannels, es = P.elemSize, me = P.rank;
@@ -833,32 +847,44 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
       if (wave == 0) {
         const uint64_t word = waitDescs(A, sh, lane, w0, w1, true, cap);
         if (sh.waitOk && (lane & 31) < n) {
-          // sources in fold order, destinations by rank
-          if (lane < 32) sh.sweep.src[(lane + n - 1 - me) % n] = word & kPtrMask;
-          else sh.sweep.dst[lane & 31] = word & kPtrMask;
-        }
-        if (sh.waitOk && lane >= n && lane < kMaxDirectRanks) {
-          sh.sweep.src[lane] = 0;
-          sh.sweep.dst[lane] = 0;
+          if (lane < 32) sh.peerSend[lane] = word & kPtrMask;
+          else sh.peerRecv[lane & 31] = word & kPtrMask;
         }
         if (sh.waitOk && lane == 0) {
           SweepGeom& g = sh.sweep;
+          const int kind = P.kind, root = P.root;
+          const bool owned = (kind == kAllReduce || kind == kReduce || kind == kBroadcast);
+          const bool folds = (kind == kAllReduce || kind == kReduce || kind == kReduceScatter);
+          const bool toAll = (kind == kAllReduce || kind == kBroadcast || kind == kAllGather);
+          const int first = (kind == kReduce) ? root + 1 : me + 1;  // rank the fold starts with
+          const uint64_t srcOff = (kind == kReduceScatter) ? (uint64_t)me * (uint64_t)count * (uint64_t)es : 0;
+          const uint64_t dstOff = (kind == kAllGather) ? (uint64_t)me * (uint64_t)count * (uint64_t)es : 0;
+          g.n = folds ? n : 1;
+          g.nd = toAll ? n : 1;
+          for (int t = 0; t < kMaxDirectRanks; t++) {
+            uint64_t sp = 0, dp = 0;
+            if (t < g.n) sp = sh.peerSend[folds ? (first + t) % n : (kind == kBroadcast ? root : me)] + srcOff;
+            if (t < g.nd) dp = sh.peerRecv[toAll ? t : (kind == kReduce ? root : me)] + dstOff;
+            g.src[t] = sp;
+            g.dst[t] = dp;
+          }
+          g.tn = owned ? n : 1;
+          g.tme = owned ? me : 0;
           g.count = count;
-          g.loop = loopElems(kAllReduce, n, C, P.chunkElems);
+          g.loop = (int64_t)C * g.tn * P.chunkElems;
           g.chunkElems = P.chunkElems;
           g.lastReal = P.lastChunkElems;
           g.L = L;
           g.T = L * C;
           g.instBase = inst * (uint64_t)(L * C);
           g.ctr = (uint64_t)(uintptr_t)P.tileCtr;
-          g.n = n;
           g.C = C;
           g.ch = ch;
           g.es = es;
           g.me = me;
           g.dtype = P.dtype;
           g.op = P.op;
-          g.pad = 0;
+          g.pad0 = g.pad1 = 0;
           sh.peersLoaded = 1;
         }
       }
@@ -933,7 +959,7 @@ __device__ __forceinline__ int runDirectAllReduce(const DaemonArgs& A, WgShared&
 }
 
 __device__ __forceinline__ int runColl(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
-  if (sh.plan.proto == kProtoDirect) return runDirectAllReduce(A, sh, ch, tid);
+  if (sh.plan.proto == kProtoDirect) return runDirect(A, sh, ch, tid);
   return runFifo(A, sh, ch, tid);
 }
 

@@ -413,11 +413,14 @@ static void planGroup(CommGroup* g) {
     g->count = (int64_t)g->countUser;
   }
   if (g->kind == kAllGather || g->kind == kReduceScatter) nBytes *= g->nRanks;
-  // protocol: the virtual ranks of an all-reduce read each other's buffers in place unless told otherwise
+  // protocol: virtual ranks read and write each other's buffers in place unless told otherwise (or too many)
   const char* proto = getenv("DFCCL_PROTO");
   const bool wantFifo = proto != nullptr && strcmp(proto, "fifo") == 0;
-  g->proto = (!wantFifo && g->kind == kAllReduce && g->nRanks >= 2 && g->nRanks <= kMaxDirectRanks) ? kProtoDirect
-                                                                                                     : kProtoFifo;
+  g->proto = (!wantFifo && g->nRanks >= 2 && g->nRanks <= kMaxDirectRanks) ? kProtoDirect : kProtoFifo;
+  // index space of the direct sweep: reduce and broadcast split the message among the ranks chunk by chunk as
+  // all-reduce does; reduce-scatter and all-gather give every rank a block of its own
+  const int geomKind = (g->proto == kProtoDirect && (g->kind == kReduce || g->kind == kBroadcast)) ? (int)kAllReduce
+                                                                                                    : g->kind;
   int64_t buff = envInt("NCCL_BUFFSIZE", 1 << 20);
   if (buff < (64 << 10)) buff = 64 << 10;
   buff = (buff / (8 * kAlignBytes)) * (8 * kAlignBytes);
@@ -445,7 +448,9 @@ static void planGroup(CommGroup* g) {
   // which is the larger of this communicator's size and the rank contexts created on the device so far.
   int sharers = g->nRanks;
   if (g->device >= 0 && g->device < 64) sharers = std::max(sharers, gLiveRankCtxs[g->device].load());
-  int maxCh = (int)envInt("NCCL_MAX_NCHANNELS", std::max(1, 256 / std::max(1, sharers)));
+  int share = std::max(1, 256 / std::max(1, sharers));
+  if (share > 8) share &= ~7;  // the launch rounds a rank's workgroups up to whole sets of 8 (one per XCD)
+  int maxCh = (int)envInt("NCCL_MAX_NCHANNELS", share);
   if (maxCh < 1) maxCh = 1;
   if (maxCh > kMaxChannels) maxCh = kMaxChannels;
   const int64_t perChannel = envInt("DFCCL_BYTES_PER_CHANNEL", (int64_t)kWgThreads * 64);
@@ -454,14 +459,14 @@ static void planGroup(CommGroup* g) {
   g->alignElems = kAlignBytes / g->elemSize;
   g->sliceElems = sliceBytes / g->elemSize;
   // a slot only has to hold the largest slice this collective will ever move
-  const int64_t real0 = realChunkElems(g->kind, g->nRanks, g->nChannels, g->chunkElems, g->alignElems,
+  const int64_t real0 = realChunkElems(geomKind, g->nRanks, g->nChannels, g->chunkElems, g->alignElems,
                                        g->count > 0 ? g->count : 1, 0);
   const int64_t maxSlice = sliceElemsFor(real0, g->slicesPerChunk, g->sliceElems);
   g->slotBytes = roundUp64(maxSlice * g->elemSize, kAlignBytes);
   g->chanStride = g->slotBytes * g->fifoSlots;
-  const int64_t loop = loopElems(g->kind, g->nRanks, g->nChannels, g->chunkElems);
+  const int64_t loop = loopElems(geomKind, g->nRanks, g->nChannels, g->chunkElems);
   g->loopsPerInstance = g->count > 0 ? divUp64(g->count, loop) : 0;
-  g->lastChunkElems = g->count > 0 ? realChunkElems(g->kind, g->nRanks, g->nChannels, g->chunkElems, g->alignElems,
+  g->lastChunkElems = g->count > 0 ? realChunkElems(geomKind, g->nRanks, g->nChannels, g->chunkElems, g->alignElems,
                                                     g->count, (g->loopsPerInstance - 1) * loop)
                                    : 0;
 }

@@ -22,8 +22,8 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(autouse=True, params=["direct", "fifo"])
 def proto(request, monkeypatch):
-    """Every test runs under both data protocols: `direct` (all-reduce reads the peers' buffers in place; the
-    other collectives still use FIFOs) and `fifo` (the reference's staged ring for everything)."""
+    """Every test runs under both data protocols: `direct` (up to 8 ranks read and write each other's buffers in
+    place) and `fifo` (the reference's staged ring)."""
     monkeypatch.setenv("DFCCL_PROTO", request.param)
     # a daemon that would otherwise stay resident leaves (and is relaunched on demand) every 10 s
     monkeypatch.setenv("DFCCL_DAEMON_MAX_MS", "10000")
@@ -57,6 +57,8 @@ def check(kind, dtype, op, n, count, root=0, seed=100, reps=1, **kw):
     with VirtualRing(n) as ring:
         ring.prepare(0, kind, count, dtype, op, root)
         ring.finalize()
+        want_proto = 1 if (os.environ.get("DFCCL_PROTO") == "direct" and 2 <= n <= 8) else 0
+        assert ring.ctxs[0].geometry(0).protocol == want_proto
         sends_np, sends, recvs = make_buffers(kind, dtype, n, count, seed, **kw)
         want = oracle_run(kind, dtype, op, geom_of(ring, 0), root, sends_np)
         for _ in range(reps):
@@ -391,3 +393,83 @@ def test_many_ranks_fall_back_to_fifo():
     # more ranks than one workgroup folds in a pass: the collective runs over FIFOs
     stats = check("all_reduce", orc.I32, orc.SUM, 12, 50000, seed=1300)
     assert stats["cqesWritten"] == 12
+
+
+def test_in_place_and_absent_buffers_of_the_other_collectives():
+    # in place as NCCL defines it: reduce-scatter receives into block `rank` of its send buffer, all-gather sends
+    # from block `rank` of its receive buffer, reduce at the root; ranks that are not the root of a reduce pass no
+    # receive buffer, ranks that are not the root of a broadcast no send buffer
+    from dfccl_amd.ring import VirtualRing
+    n, count, root = 4, 30011, 1
+    with VirtualRing(n) as ring:
+        ring.prepare(0, "reduce_scatter", count, orc.F32, orc.SUM)
+        ring.prepare(1, "all_gather", count, orc.F16)
+        ring.prepare(2, "reduce", count, orc.BF16, orc.SUM, root)
+        ring.prepare(3, "broadcast", count, orc.I8, root=root)
+        ring.finalize()
+        # reduce-scatter
+        sends_np, sends, _ = make_buffers("reduce_scatter", orc.F32, n, count, 2100)
+        want = orc.reduce_scatter(orc.F32, orc.SUM, geom_of(ring, 0), sends_np)
+        ring.run(0, sends, [sends[r][r * count:(r + 1) * count] for r in range(n)], timeout=30)
+        for r in range(n):
+            assert np.array_equal(to_np(orc.F32, sends[r][r * count:(r + 1) * count]), want[r]), ("reduce_scatter", r)
+        # all-gather
+        sends_np, _, recvs = make_buffers("all_gather", orc.F16, n, count, 2200)
+        for r in range(n):
+            recvs[r][r * count:(r + 1) * count].copy_(to_gpu(orc.F16, sends_np[r]))
+        torch.cuda.current_stream().synchronize()
+        want = orc.all_gather(orc.F16, geom_of(ring, 1), sends_np)
+        ring.run(1, [recvs[r][r * count:(r + 1) * count] for r in range(n)], recvs, timeout=30)
+        for r in range(n):
+            assert np.array_equal(to_np(orc.F16, recvs[r]), want[r]), ("all_gather", r)
+        # reduce: in place at the root, no receive buffer elsewhere
+        sends_np, sends, _ = make_buffers("reduce", orc.BF16, n, count, 2300)
+        want = orc.reduce(orc.BF16, orc.SUM, geom_of(ring, 2), root, sends_np)
+        ring.run(2, sends, [sends[r] if r == root else None for r in range(n)], timeout=30)
+        assert np.array_equal(to_np(orc.BF16, sends[root]), want[root])
+        for r in range(n):
+            if r != root:  # the other ranks' send buffers are untouched
+                assert np.array_equal(to_np(orc.BF16, sends[r]), sends_np[r])
+        # broadcast: no send buffer except at the root
+        sends_np, sends, recvs = make_buffers("broadcast", orc.I8, n, count, 2400)
+        ring.run(3, [sends[r] if r == root else None for r in range(n)], recvs, timeout=30)
+        for r in range(n):
+            assert np.array_equal(to_np(orc.I8, recvs[r]), sends_np[root]), ("broadcast", r)
+
+
+@pytest.mark.parametrize("kind,dtype,op", [("reduce_scatter", orc.F16, orc.SUM), ("reduce", orc.F32, orc.SUM),
+                                           ("reduce", orc.BF16, orc.PROD), ("all_gather", orc.I8, orc.SUM),
+                                           ("broadcast", orc.F16, orc.SUM)])
+@pytest.mark.parametrize("n,count", [(8, 3_000_017), (5, 999_999), (2, 12_345_678)])
+def test_other_collectives_large_and_ragged(kind, dtype, op, n, count):
+    # several channels and loops, sizes that are no multiple of anything (all-gather then writes at offsets that
+    # rule out 128-bit accesses), a root in the middle
+    if kind in ("all_gather", "reduce_scatter"):
+        count //= n
+    check(kind, dtype, op, n, count, root=n // 2, seed=2500 + n, small_ints=(op == orc.PROD))
+
+
+def test_other_collectives_disordered_submission(proto):
+    # the four other collectives registered side by side, every rank submitting them in its own order
+    from dfccl_amd.ring import VirtualRing
+    n, count = 4, 70_001
+    kinds = ["reduce_scatter", "all_gather", "reduce", "broadcast", "all_reduce"] * 3
+    rng = np.random.default_rng(26)
+    with VirtualRing(n) as ring:
+        for cid, kind in enumerate(kinds):
+            ring.prepare(cid, kind, count, orc.F32, orc.SUM, root=cid % n)
+        ring.finalize()
+        bufs, wants = [], []
+        for cid, kind in enumerate(kinds):
+            sends_np, sends, recvs = make_buffers(kind, orc.F32, n, count, 2600 + 10 * cid)
+            bufs.append((sends, recvs))
+            wants.append(oracle_run(kind, orc.F32, orc.SUM, geom_of(ring, cid), cid % n, sends_np))
+        for r in range(n):
+            for cid in rng.permutation(len(kinds)):
+                ring.submit(r, int(cid), bufs[cid][0][r], bufs[cid][1][r])
+        ring.wait([(r, cid) for r in range(n) for cid in range(len(kinds))], timeout=60)
+        for cid, kind in enumerate(kinds):
+            for r in range(n):
+                if kind == "reduce" and r != cid % n:
+                    continue
+                assert np.array_equal(to_np(orc.F32, bufs[cid][1][r]), wants[cid][r]), (cid, kind, r)
