@@ -151,6 +151,20 @@ def bench_buckets():
     return out
 
 
+def bench_other_collectives():
+    """Reduce-scatter, all-gather, reduce and broadcast over 8 virtual ranks (bf16; 8 MiB per rank block for the
+    first two, 64 MiB messages for the other two) through the daemon, direct protocol. GB/s on the bytes the direct
+    protocol moves (every input read once, every output written once)."""
+    out = {}
+    for kind in ("reduce_scatter", "all_gather", "reduce", "broadcast"):
+        nbytes = (8 << 20) if kind in ("reduce_scatter", "all_gather") else (64 << 20)
+        r = run_native(["collective", "--kind", kind, "--ranks", 8, "--bytes", nbytes, "--dtype", "bf16",
+                        "--iters", 10])
+        out[kind] = {"ms": r["best_ms"], "traffic_GBps": r["direct_traffic_GBps"], "protocol": r["protocol"],
+                     "channels": r["channels"], "count_bytes": r["count_bytes"], "correct": r["correct"]}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -203,6 +217,7 @@ def main():
         line["sqe_to_cqe_latency"] = bench_latency()
         line["disordered_small_collectives"] = bench_disordered()
         line["gradient_buckets"] = bench_buckets()
+        line["other_collectives"] = bench_other_collectives()
     if not args.skip_cpu:
         line["cpu_baseline"] = bench_cpu_baseline()
     print(json.dumps(line))

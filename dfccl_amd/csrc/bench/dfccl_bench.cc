@@ -6,6 +6,7 @@
 //   dfccl_bench disorder  --ranks 4 --colls 256 --min-bytes 4096 --max-bytes 4194304
 //   dfccl_bench allreduce --ranks 8 --bytes 67108864 --dtype bf16 --iters 10
 //   dfccl_bench buckets   --ranks 4 --colls 40 --elems 25000000 --dtype int32
+//   dfccl_bench collective --kind reduce_scatter|all_gather|reduce|broadcast --ranks 8 --bytes 67108864 --dtype bf16
 //
 // Every mode prints one JSON object on stdout.  Inputs are small integers
 // (rank + 1) so that every reduction is exact in every dtype and the outputs can
@@ -52,7 +53,7 @@ struct Args {
   std::string mode;
   int ranks = 4, colls = 256, iters = 1000, warmup = 50;
   size_t bytes = 4096, minBytes = 4096, maxBytes = 4 << 20, elems = 25000000;
-  std::string dtype = "fp16";
+  std::string dtype = "fp16", kind = "reduce_scatter";
   uint64_t seed = 3;
   int timeoutS = 60;
 };
@@ -159,6 +160,21 @@ struct World {
     for (int r = 0; r < n; r++) {
       NK(ncclCommInitRank(&c[r], n, id, r));
       NK(ofcclPrepareAllReduce(count, (ncclDataType_t)dt, ncclSum, c[r], collId, ctx[r]));
+    }
+    comms.push_back(c);
+  }
+  // kind: 1 reduce-scatter, 2 all-gather, 3 reduce, 4 broadcast (count as the respective Prepare call takes it)
+  void prepareKind(int kind, int collId, size_t count, int dt, int root) {
+    ncclUniqueId id;
+    NK(ncclGetUniqueId(&id));
+    std::vector<ncclComm_t> c(n);
+    for (int r = 0; r < n; r++) {
+      NK(ncclCommInitRank(&c[r], n, id, r));
+      const ncclDataType_t t = (ncclDataType_t)dt;
+      if (kind == 1) NK(ofcclPrepareReduceScatter(count, t, ncclSum, c[r], collId, ctx[r]));
+      else if (kind == 2) NK(ofcclPrepareAllGather(count, t, c[r], collId, ctx[r]));
+      else if (kind == 3) NK(ofcclPrepareReduce(count, t, ncclSum, root, c[r], collId, ctx[r]));
+      else NK(ofcclPrepareBroadcast(count, t, root, c[r], collId, ctx[r]));
     }
     comms.push_back(c);
   }
@@ -408,9 +424,79 @@ static int runBuckets(const Args& a, bool single) {
   return ok ? 0 : 1;
 }
 
+// ---- collective: one large reduce-scatter / all-gather / reduce / broadcast ----------------------
+static int runCollective(const Args& a) {
+  const int n = a.ranks, dt = dtypeCode(a.dtype), es = dtypeSize(dt), root = 0;
+  const int kind = a.kind == "reduce_scatter" ? 1 : a.kind == "all_gather" ? 2 : a.kind == "reduce" ? 3 : a.kind == "broadcast" ? 4 : 0;
+  if (kind == 0) { fprintf(stderr, "unknown --kind %s\n", a.kind.c_str()); return 2; }
+  const size_t count = a.bytes / es;
+  const size_t sendElems = kind == 1 ? count * n : count, recvElems = kind == 2 ? count * n : count;
+  World w(n);
+  w.prepareKind(kind, 0, count, dt, root);
+  w.finalize();
+  dfcclCollGeometry geom{};
+  NK(dfcclGetCollGeometry(w.ctx[0], 0, &geom));
+  std::vector<void*> send(n), recv(n);
+  for (int r = 0; r < n; r++) {
+    CK(hipMalloc(&send[r], sendElems * es));
+    CK(hipMalloc(&recv[r], recvElems * es));
+    fillBuffer(send[r], sendElems, dt, r + 1);
+    fillBuffer(recv[r], recvElems, dt, 0);
+  }
+  CK(hipStreamSynchronize(nullptr));
+  std::vector<Flag> flags(n);
+  SpinBarrier bar(n);
+  std::atomic<int> failed{0};
+  const int total = a.iters + 2;
+  std::vector<uint64_t> tStart(total);
+  std::vector<std::atomic<uint64_t>> endNs(total);
+  for (auto& e : endNs) e.store(0);
+  std::vector<std::thread> th;
+  for (int r = 0; r < n; r++) {
+    th.emplace_back([&, r] {
+      CK(hipSetDevice(0));
+      for (int it = 0; it < total && !failed.load(); it++) {
+        flags[r].done.store(0);
+        bar.wait();
+        if (r == 0) tStart[it] = nowNs();
+        if (kind == 1) NK(ofcclRunReduceScatter(send[r], recv[r], 0, onDone, &flags[r], w.ctx[r]));
+        else if (kind == 2) NK(ofcclRunAllGather(send[r], recv[r], 0, onDone, &flags[r], w.ctx[r]));
+        else if (kind == 3) NK(ofcclRunReduce(send[r], recv[r], 0, onDone, &flags[r], w.ctx[r]));
+        else NK(ofcclRunBroadcast(send[r], recv[r], 0, onDone, &flags[r], w.ctx[r]));
+        if (!waitFlag(flags[r], a.timeoutS)) { failed.store(1); fprintf(stderr, "rank %d timed out\n", r); return; }
+        uint64_t t = nowNs(), prev = endNs[it].load();
+        while (prev < t && !endNs[it].compare_exchange_weak(prev, t)) {}
+        bar.wait();
+      }
+    });
+  }
+  for (auto& t : th) t.join();
+  bool ok = !failed.load();
+  std::vector<double> ms;
+  for (int it = 2; it < total && ok; it++) ms.push_back((double)(endNs[it].load() - tStart[it]) / 1e6);
+  std::vector<char> scratch;
+  const int sum = n * (n + 1) / 2;
+  for (int r = 0; r < n && ok; r++) {
+    if (kind == 1) ok = verifyBuffer(recv[r], count, dt, sum, scratch);
+    else if (kind == 2) { for (int b = 0; b < n && ok; b++) ok = verifyBuffer((char*)recv[r] + (size_t)b * count * es, count, dt, b + 1, scratch); }
+    else if (kind == 3) { if (r == root) ok = verifyBuffer(recv[r], count, dt, sum, scratch); }
+    else ok = verifyBuffer(recv[r], count, dt, root + 1, scratch);
+  }
+  w.destroy();
+  const double best = ms.empty() ? 0 : *std::min_element(ms.begin(), ms.end());
+  // HBM bytes the direct protocol moves, all ranks together (every input element read once, every output written once)
+  const double B = (double)count * es;
+  const double moved = kind == 1 ? 1.0 * n * n * B + n * B : kind == 2 ? n * B + 1.0 * n * n * B : kind == 3 ? n * B + B : B + n * B;
+  printf("{\"mode\": \"collective\", \"kind\": \"%s\", \"ranks\": %d, \"dtype\": \"%s\", \"count_bytes\": %zu, \"protocol\": \"%s\", "
+         "\"channels\": %d, \"iters\": %d, \"correct\": %s, \"best_ms\": %.4f, \"median_ms\": %.4f, \"direct_traffic_GBps\": %.1f}\n",
+         a.kind.c_str(), n, a.dtype.c_str(), count * es, geom.protocol == 1 ? "direct" : "fifo", geom.nChannels, a.iters,
+         ok ? "true" : "false", best, pct(ms, 0.5), best > 0 ? moved / (best * 1e-3) / 1e9 : 0);
+  return ok ? 0 : 1;
+}
+
 int main(int argc, char** argv) {
   if (argc < 2) {
-    fprintf(stderr, "usage: dfccl_bench latency|disorder|allreduce|buckets [options]\n");
+    fprintf(stderr, "usage: dfccl_bench latency|disorder|allreduce|buckets|collective [options]\n");
     return 2;
   }
   Args a;
@@ -426,6 +512,7 @@ int main(int argc, char** argv) {
     else if (k == "--max-bytes") a.maxBytes = strtoull(v.c_str(), nullptr, 10);
     else if (k == "--elems") a.elems = strtoull(v.c_str(), nullptr, 10);
     else if (k == "--dtype") a.dtype = v;
+    else if (k == "--kind") a.kind = v;
     else if (k == "--seed") a.seed = strtoull(v.c_str(), nullptr, 10);
     else if (k == "--timeout") a.timeoutS = atoi(v.c_str());
     else { fprintf(stderr, "unknown option %s\n", k.c_str()); return 2; }
@@ -435,6 +522,7 @@ int main(int argc, char** argv) {
   if (a.mode == "disorder") return runDisorder(a);
   if (a.mode == "allreduce") return runBuckets(a, true);
   if (a.mode == "buckets") return runBuckets(a, false);
+  if (a.mode == "collective") return runCollective(a);
   fprintf(stderr, "unknown mode %s\n", a.mode.c_str());
   return 2;
 }
