@@ -13,6 +13,8 @@
 // be verified element by element on the host.
 #include <hip/hip_runtime.h>
 
+#include <signal.h>
+
 #include <algorithm>
 #include <atomic>
 #include <chrono>
@@ -55,7 +57,7 @@ struct Args {
   size_t bytes = 4096, minBytes = 4096, maxBytes = 4 << 20, elems = 25000000;
   std::string dtype = "fp16", kind = "reduce_scatter";
   uint64_t seed = 3;
-  int timeoutS = 60;
+  int timeoutS = 20;
 };
 
 static int dtypeCode(const std::string& s) {
@@ -113,6 +115,11 @@ static int onDone(int, void* arg) {
   return 0;
 }
 
+// Set when a rank has given up waiting (or the process was told to stop): every wait in the driver ends then, so
+// that the run is torn down in order (a driver that is killed while the daemon kernel is resident leaves the GPU
+// with a kernel nobody will ever stop).
+static std::atomic<int> gGiveUp{0};
+
 struct SpinBarrier {
   std::atomic<int> count{0};
   std::atomic<int> gen{0};
@@ -124,7 +131,7 @@ struct SpinBarrier {
       count.store(0, std::memory_order_release);
       gen.fetch_add(1, std::memory_order_acq_rel);
     } else {
-      while (gen.load(std::memory_order_acquire) == g) __builtin_ia32_pause();
+      while (gen.load(std::memory_order_acquire) == g && !gGiveUp.load(std::memory_order_acquire)) __builtin_ia32_pause();
     }
   }
 };
@@ -141,7 +148,10 @@ static bool waitFlag(Flag& f, int timeoutS) {
   uint64_t spins = 0;
   while (!f.done.load(std::memory_order_acquire)) {
     __builtin_ia32_pause();
-    if ((++spins & 0xffff) == 0 && nowNs() > deadline) return false;
+    if ((++spins & 0xfff) == 0 && (gGiveUp.load(std::memory_order_acquire) || nowNs() > deadline)) {
+      gGiveUp.store(1, std::memory_order_release);
+      return false;
+    }
   }
   return true;
 }
@@ -192,6 +202,18 @@ struct World {
     }
     return t;
   }
+  // what the daemon has done so far, rank by rank (printed when a run is given up)
+  void report() {
+    for (int r = 0; r < n; r++) {
+      dfcclStats s{};
+      if (dfcclGetStats(ctx[r], &s) != ncclSuccess) continue;
+      fprintf(stderr, "rank %d: sqes read %llu, cqes written %llu, ctx saves %llu, loads %llu, slices moved %llu, "
+              "voluntary quits %llu, launches %llu\n", r, (unsigned long long)s.sqesRead,
+              (unsigned long long)s.cqesWritten, (unsigned long long)s.ctxSaves, (unsigned long long)s.ctxLoads,
+              (unsigned long long)s.slicesMoved, (unsigned long long)s.voluntaryQuits,
+              (unsigned long long)s.daemonLaunches);
+    }
+  }
   void destroy() {
     for (int r = 0; r < n; r++) NK(ofcclDestroy(ctx[r]));
     for (auto& c : comms)
@@ -223,7 +245,7 @@ static int runLatency(const Args& a) {
   for (int r = 0; r < n; r++) {
     th.emplace_back([&, r] {
       CK(hipSetDevice(0));
-      for (int it = 0; it < total && !failed.load(); it++) {
+      for (int it = 0; it < total && !failed.load() && !gGiveUp.load(); it++) {
         flags[r].done.store(0, std::memory_order_release);
         bar.wait();
         NK(ofcclRunAllReduce(send[r], recv[r], 0, onDone, &flags[r], w.ctx[r]));
@@ -236,7 +258,8 @@ static int runLatency(const Args& a) {
   }
   for (auto& t : th) t.join();
   std::vector<char> scratch;
-  bool ok = !failed.load();
+  bool ok = !failed.load() && !gGiveUp.load();
+  if (!ok) w.report();
   for (int r = 0; r < n && ok; r++) ok = verifyBuffer(recv[r], count, dt, n * (n + 1) / 2, scratch);
   std::vector<double> all;
   for (auto& v : lat) all.insert(all.end(), v.begin(), v.end());
@@ -308,7 +331,8 @@ static int runDisorder(const Args& a) {
     });
   }
   for (auto& t : th) t.join();
-  bool ok = !failed.load();
+  bool ok = !failed.load() && !gGiveUp.load();
+  if (!ok) w.report();
   std::vector<double> all, small;
   for (int r = 0; r < n && ok; r++)
     for (int c = 0; c < nc; c++) {
@@ -368,7 +392,7 @@ static int runBuckets(const Args& a, bool single) {
   for (int r = 0; r < n; r++) {
     th.emplace_back([&, r] {
       CK(hipSetDevice(0));
-      for (int it = 0; it < total && !failed.load(); it++) {
+      for (int it = 0; it < total && !failed.load() && !gGiveUp.load(); it++) {
         for (int c = 0; c < nc; c++) flags[(size_t)r * nc + c].done.store(0);
         bar.wait();
         if (r == 0) tStart[it] = nowNs();
@@ -390,7 +414,8 @@ static int runBuckets(const Args& a, bool single) {
     });
   }
   for (auto& t : th) t.join();
-  bool ok = !failed.load();
+  bool ok = !failed.load() && !gGiveUp.load();
+  if (!ok) w.report();
   for (int it = (single ? 2 : 1); it < total && ok; it++) ms.push_back((double)(endNs[it].load() - tStart[it]) / 1e6);
   std::vector<char> scratch;
   for (int c = 0; c < nc && ok; c += std::max(1, nc / 4))
@@ -455,7 +480,7 @@ static int runCollective(const Args& a) {
   for (int r = 0; r < n; r++) {
     th.emplace_back([&, r] {
       CK(hipSetDevice(0));
-      for (int it = 0; it < total && !failed.load(); it++) {
+      for (int it = 0; it < total && !failed.load() && !gGiveUp.load(); it++) {
         flags[r].done.store(0);
         bar.wait();
         if (r == 0) tStart[it] = nowNs();
@@ -471,7 +496,8 @@ static int runCollective(const Args& a) {
     });
   }
   for (auto& t : th) t.join();
-  bool ok = !failed.load();
+  bool ok = !failed.load() && !gGiveUp.load();
+  if (!ok) w.report();
   std::vector<double> ms;
   for (int it = 2; it < total && ok; it++) ms.push_back((double)(endNs[it].load() - tStart[it]) / 1e6);
   std::vector<char> scratch;
@@ -494,7 +520,15 @@ static int runCollective(const Args& a) {
   return ok ? 0 : 1;
 }
 
+static void onSignal(int sig) {
+  // end the waits; the modes then tear the rank contexts down, which stops the daemon kernel
+  gGiveUp.store(1, std::memory_order_release);
+  (void)sig;
+}
+
 int main(int argc, char** argv) {
+  signal(SIGTERM, onSignal);
+  signal(SIGINT, onSignal);
   if (argc < 2) {
     fprintf(stderr, "usage: dfccl_bench latency|disorder|allreduce|buckets|collective [options]\n");
     return 2;

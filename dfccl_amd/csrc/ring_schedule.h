@@ -128,6 +128,62 @@ DFCCL_HD StepDesc describeStep(int kind, int n, int rank, int root, int nChannel
   return d;
 }
 
+// ---- direct protocol (virtual ranks read and write each other's buffers in place) -------------------
+//
+// Host-side statement of the roles and the tile geometry (used by the planner and by the CPU tests, which run
+// every rank's share through it and compare with the oracle); the daemon kernel evaluates the same expressions
+// in place (runDirect, sweepFoldN).
+//
+// Every rank does a share of the collective: it folds `nSrc` send buffers (in the order in which the ring would
+// have accumulated those elements) and stores the result into `nDst` receive buffers.  The share is a set of
+// tiles: the index space [0, count) is cut into loops of nChannels * tn chunks, and tile t of a rank is chunk
+// number tme of channel slot t % nChannels in loop t / nChannels.
+//   all-reduce      tn = n, tme = me (the chunks the ring would finish at me);  in[me+1], ..., in[me] -> all
+//   reduce          tn = n, tme = me;  in[root+1], ..., in[root] -> the root's receive buffer
+//   broadcast       tn = n, tme = me;  the root's send buffer -> all
+//   reduce-scatter  tn = 1 (block me of every send buffer is all mine);  in[me+1], ..., in[me] -> mine
+//   all-gather      tn = 1;  my send buffer -> block me of all
+struct DirectRole {
+  int nSrc, nDst;
+  int firstSrc;       // rank of source 0; source t is rank (firstSrc + t) % n
+  int onlyDst;        // rank of the single destination, -1: destination k is rank k
+  int tn, tme;
+  int64_t srcOff;     // elements added to every source / destination pointer
+  int64_t dstOff;
+};
+
+DFCCL_HD DirectRole directRole(int kind, int n, int me, int root, int64_t count) {
+  DirectRole r;
+  const bool folds = (kind == kAllReduce || kind == kReduce || kind == kReduceScatter);
+  const bool toAll = (kind == kAllReduce || kind == kBroadcast || kind == kAllGather);
+  const bool owned = (kind == kAllReduce || kind == kReduce || kind == kBroadcast);
+  r.nSrc = folds ? n : 1;
+  r.nDst = toAll ? n : 1;
+  r.firstSrc = folds ? ((kind == kReduce ? root : me) + 1) % n : (kind == kBroadcast ? root : me);
+  r.onlyDst = toAll ? -1 : (kind == kReduce ? root : me);
+  r.tn = owned ? n : 1;
+  r.tme = owned ? me : 0;
+  r.srcOff = (kind == kReduceScatter) ? (int64_t)me * count : 0;
+  r.dstOff = (kind == kAllGather) ? (int64_t)me * count : 0;
+  return r;
+}
+
+// Geometry kind whose loop / chunk arithmetic (loopElems, realChunkElems) the direct protocol uses for `kind`:
+// a loop of all-reduce holds nChannels * n chunks, a loop of the others nChannels.
+DFCCL_HD int directGeomKind(int kind) { return (kind == kReduce || kind == kBroadcast) ? (int)kAllReduce : kind; }
+
+// Tile t of a rank: offset and length in elements (length <= 0: nothing there).  lastReal is the chunk size of
+// the last loop (realChunkElems at its start), every other loop uses the nominal chunk.
+DFCCL_HD void directTile(int64_t tile, int nChannels, int64_t loops, int64_t chunkElems, int64_t lastReal, int tn,
+                         int tme, int64_t count, int64_t* off, int64_t* nelem) {
+  // (tile numbers fit 32 bits: 64-bit divisions are long instruction sequences on the GPU)
+  const int64_t l = (int64_t)((uint32_t)tile / (uint32_t)nChannels), slot = (int64_t)((uint32_t)tile % (uint32_t)nChannels);
+  const int64_t real = (l == loops - 1) ? lastReal : chunkElems;
+  const int64_t o = l * ((int64_t)nChannels * tn * chunkElems) + (slot * tn + tme) * real;
+  *off = o;
+  *nelem = (count - o < real) ? count - o : real;
+}
+
 // Channels (workgroups per rank) for a collective of nBytes: as many as allowed,
 // shrunk until each gets at least bytesPerChannel (the thread-count shrink rule
 // of src/enqueue_ofccl.cc:133-137 with a fixed workgroup size).

@@ -419,8 +419,7 @@ static void planGroup(CommGroup* g) {
   g->proto = (!wantFifo && g->nRanks >= 2 && g->nRanks <= kMaxDirectRanks) ? kProtoDirect : kProtoFifo;
   // index space of the direct sweep: reduce and broadcast split the message among the ranks chunk by chunk as
   // all-reduce does; reduce-scatter and all-gather give every rank a block of its own
-  const int geomKind = (g->proto == kProtoDirect && (g->kind == kReduce || g->kind == kBroadcast)) ? (int)kAllReduce
-                                                                                                    : g->kind;
+  const int geomKind = (g->proto == kProtoDirect) ? directGeomKind(g->kind) : g->kind;
   int64_t buff = envInt("NCCL_BUFFSIZE", 1 << 20);
   if (buff < (64 << 10)) buff = 64 << 10;
   buff = (buff / (8 * kAlignBytes)) * (8 * kAlignBytes);

@@ -7,6 +7,7 @@
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <utility>
 #include <vector>
 
 #include "../dfccl_amd/csrc/ring_schedule.h"
@@ -111,4 +112,50 @@ extern "C" int sim_plan_channels(int64_t nBytes, int maxChannels, int64_t bytesP
 extern "C" uint64_t sim_cqe_encode(unsigned blk, unsigned cnt, unsigned coll) { return cqeEncode(blk, cnt, coll); }
 extern "C" void sim_cqe_decode(uint64_t v, unsigned* blk, unsigned* cnt, unsigned* coll) {
   *blk = cqeBlk(v); *cnt = cqeCnt(v); *coll = cqeCollId(v);
+}
+
+// The direct protocol on the host: every rank's share is processed tile by tile, in the order given by
+// `order` (a permutation seed: tiles may be taken by any workgroup at any time on the device), with the roles
+// and the tile geometry of ring_schedule.h and the oracle's element arithmetic.  Returns the number of elements
+// written, or -1 if a destination element was written twice.
+extern "C" int64_t sim_direct(int kind, int dtype, int op, int n, int nChannels, int64_t chunkElems, int64_t alignElems,
+                              int64_t count, int root, const void* const* send, void* const* recv, uint64_t order) {
+  int es = orc_type_size(dtype);
+  if (kind == kAllGather || kind == kBroadcast) { count *= es; dtype = ORC_I8; es = 1; }
+  const int gk = directGeomKind(kind);
+  const int64_t loop = loopElems(gk, n, nChannels, chunkElems);
+  const int64_t loops = count > 0 ? (count + loop - 1) / loop : 0;
+  const int64_t lastReal = count > 0 ? realChunkElems(gk, n, nChannels, chunkElems, alignElems, count, (loops - 1) * loop) : 0;
+  const int64_t tiles = loops * nChannels;
+  int64_t written = 0;
+  // snapshot of the inputs: in place runs read what the instance started with only where the device does too
+  // (each element is read by the one thread that writes it), so reading the live buffers is the faithful model
+  std::vector<std::pair<int, int64_t>> work;  // (rank, tile)
+  for (int r = 0; r < n; r++)
+    for (int64_t t = 0; t < tiles; t++) work.push_back({r, t});
+  uint64_t s = order * 0x9E3779B97F4A7C15ull + 1;
+  for (size_t i = work.size(); i > 1; i--) {  // Fisher-Yates with splitmix steps
+    s += 0x9E3779B97F4A7C15ull;
+    uint64_t z = s; z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull; z = (z ^ (z >> 27)) * 0x94D049BB133111EBull; z ^= z >> 31;
+    std::swap(work[i - 1], work[(size_t)(z % i)]);
+  }
+  std::vector<char> tmp;
+  for (auto& w : work) {
+    const int me = w.first;
+    const DirectRole role = directRole(kind, n, me, root, count);
+    int64_t off, nelem;
+    directTile(w.second, nChannels, loops, chunkElems, lastReal, role.tn, role.tme, count, &off, &nelem);
+    if (nelem <= 0) continue;
+    std::vector<const void*> srcs(role.nSrc);
+    for (int t = 0; t < role.nSrc; t++)
+      srcs[t] = (const char*)send[(role.firstSrc + t) % n] + (role.srcOff + off) * es;
+    tmp.resize((size_t)nelem * es);
+    orc_reduce_copy(dtype, op, role.nSrc, srcs.data(), tmp.data(), (size_t)nelem);
+    for (int k = 0; k < role.nDst; k++) {
+      const int dr = role.onlyDst < 0 ? k : role.onlyDst;
+      memcpy((char*)recv[dr] + (role.dstOff + off) * es, tmp.data(), (size_t)nelem * es);
+      written += nelem;
+    }
+  }
+  return written;
 }

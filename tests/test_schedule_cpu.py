@@ -29,6 +29,8 @@ def sim(tmp_path_factory):
     vpp = ctypes.POINTER(ctypes.c_void_p)
     lib.sim_collective.argtypes = [ctypes.c_int] * 5 + [ctypes.c_int64] * 3 + [ctypes.c_int] * 2 + \
         [ctypes.c_int64, ctypes.c_int, vpp, vpp, ctypes.POINTER(ctypes.c_int64)]
+    lib.sim_direct.argtypes = [ctypes.c_int] * 5 + [ctypes.c_int64] * 3 + [ctypes.c_int, vpp, vpp, ctypes.c_uint64]
+    lib.sim_direct.restype = ctypes.c_int64
     lib.sim_plan_channels.argtypes = [ctypes.c_int64, ctypes.c_int, ctypes.c_int64]
     lib.sim_cqe_encode.argtypes = [ctypes.c_uint] * 3
     lib.sim_cqe_encode.restype = ctypes.c_uint64
@@ -135,3 +137,85 @@ def test_cqe_encoding_equals_oracle(sim):
         b, c, i = ctypes.c_uint(), ctypes.c_uint(), ctypes.c_uint()
         sim.sim_cqe_decode(v, ctypes.byref(b), ctypes.byref(c), ctypes.byref(i))
         assert (b.value, c.value, i.value) == (blk, cnt, coll)
+
+
+# ---- direct protocol: roles and tile geometry of ring_schedule.h against the oracle ---------------------------
+
+def run_direct(sim, kind, dtype, op, n, C, chunk, align, count, root, sends, recvs, order):
+    return sim.sim_direct(KIND[kind], dtype, op, n, C, chunk, align, count, root, orc._ptrs(sends), orc._ptrs(recvs),
+                          order)
+
+
+def kind_buffers(kind, dtype, n, count, seed, **kw):
+    send_len = count * n if kind == "reduce_scatter" else count
+    recv_len = count * n if kind == "all_gather" else count
+    sends = [datagen.make(dtype, seed + r, send_len, **kw) for r in range(n)]
+    recvs = [np.zeros(recv_len, dtype=sends[0].dtype) for _ in range(n)]
+    return sends, recvs
+
+
+def oracle_kind(kind, dtype, op, g, root, sends):
+    if kind == "all_reduce":
+        return orc.all_reduce(dtype, op, g, sends)
+    if kind == "reduce_scatter":
+        return orc.reduce_scatter(dtype, op, g, sends)
+    if kind == "all_gather":
+        return orc.all_gather(dtype, g, sends)
+    if kind == "reduce":
+        return orc.reduce(dtype, op, g, root, sends)
+    return orc.broadcast(dtype, g, root, sends)
+
+
+DIRECT_CASES = [(2, 1, 64, 16, 1000), (3, 2, 64, 16, 1000), (4, 1, 128, 32, 37), (4, 3, 32, 16, 5000),
+                (8, 2, 64, 64, 4096), (8, 4, 256, 64, 100003), (5, 1, 16, 16, 3), (2, 2, 512, 128, 513),
+                (4, 64, 4096, 512, 1 << 20), (7, 5, 48, 16, 12345)]
+
+
+@pytest.mark.parametrize("kind", list(KIND))
+@pytest.mark.parametrize("n,C,chunk,align,count", DIRECT_CASES)
+@pytest.mark.parametrize("dtype,op", [(orc.F32, orc.SUM), (orc.BF16, orc.SUM), (orc.I8, orc.MIN)])
+def test_direct_protocol_roles_and_tiles_match_oracle(sim, kind, n, C, chunk, align, count, dtype, op):
+    root = (n - 1) // 2
+    if kind in ("reduce_scatter", "all_gather"):
+        count = max(1, count // n)
+    sends, recvs = kind_buffers(kind, dtype, n, count, 40)
+    want = oracle_kind(kind, dtype, op, orc.Geom(n, C, chunk, align), root, sends)
+    for order in (0, 7):  # two different orders in which the tiles are taken
+        for t in recvs:
+            t[...] = 0
+        written = run_direct(sim, kind, dtype, op, n, C, chunk, align, count, root, sends, recvs, order)
+        # every destination element is written exactly once
+        expect = {"all_reduce": n * count, "reduce_scatter": n * count, "all_gather": n * n * count,
+                  "reduce": count, "broadcast": n * count}[kind]
+        if kind in ("all_gather", "broadcast"):
+            expect *= orc.TYPE_SIZE[dtype]  # these run as bytes
+        assert written == expect
+        for r in range(n):
+            if kind == "reduce" and r != root:
+                assert not recvs[r].any()
+                continue
+            assert np.array_equal(recvs[r], want[r]), (kind, order, r)
+
+
+@pytest.mark.parametrize("kind", ["all_reduce", "reduce_scatter", "all_gather", "reduce", "broadcast"])
+def test_direct_protocol_in_place(sim, kind):
+    n, C, chunk, align, count, root, dtype = 4, 2, 64, 16, 3000, 1, orc.F32
+    sends, _ = kind_buffers(kind, dtype, n, count, 70)
+    want = oracle_kind(kind, dtype, orc.SUM, orc.Geom(n, C, chunk, align), root, [s.copy() for s in sends])
+    if kind == "reduce_scatter":
+        bufs = [s.copy() for s in sends]
+        recvs = [bufs[r][r * count:(r + 1) * count] for r in range(n)]
+        run_direct(sim, kind, dtype, orc.SUM, n, C, chunk, align, count, root, bufs, recvs, 3)
+    elif kind == "all_gather":
+        recvs = [np.zeros(count * n, dtype=sends[0].dtype) for _ in range(n)]
+        for r in range(n):
+            recvs[r][r * count:(r + 1) * count] = sends[r]
+        run_direct(sim, kind, dtype, orc.SUM, n, C, chunk, align, count, root,
+                   [recvs[r][r * count:(r + 1) * count] for r in range(n)], recvs, 3)
+    else:
+        recvs = [s.copy() for s in sends]
+        run_direct(sim, kind, dtype, orc.SUM, n, C, chunk, align, count, root, recvs, recvs, 3)
+    for r in range(n):
+        if kind == "reduce" and r != root:
+            continue
+        assert np.array_equal(recvs[r], want[r]), (kind, r)
