@@ -188,7 +188,7 @@ def test_disordered_submission_completes_and_is_correct():
             for r in range(n):
                 cid = int(orders[r][i])
                 ring.submit(r, cid, data[cid][1][r], data[cid][2][r])
-        ring.wait([(r, cid) for r in range(n) for cid in range(ncoll)], timeout=60)
+        ring.wait([(r, cid) for r in range(n) for cid in range(ncoll)], timeout=40)
         for cid in range(ncoll):
             want = orc.all_reduce(orc.F16, orc.SUM, geom_of(ring, cid), data[cid][0])
             for r in range(n):
@@ -212,7 +212,7 @@ def test_rank_by_rank_submission_needs_preemption():
             for cid in order:
                 ring.submit(r, cid, data[cid][1][r], data[cid][2][r])
             time.sleep(0.02)
-        ring.wait([(r, cid) for r in range(n) for cid in range(ncoll)], timeout=60)
+        ring.wait([(r, cid) for r in range(n) for cid in range(ncoll)], timeout=40)
         for cid in range(ncoll):
             want = sum(s.astype(np.int64) for s in data[cid][0]).astype(np.int32)
             for r in range(n):
@@ -467,7 +467,7 @@ def test_other_collectives_disordered_submission(proto):
         for r in range(n):
             for cid in rng.permutation(len(kinds)):
                 ring.submit(r, int(cid), bufs[cid][0][r], bufs[cid][1][r])
-        ring.wait([(r, cid) for r in range(n) for cid in range(len(kinds))], timeout=60)
+        ring.wait([(r, cid) for r in range(n) for cid in range(len(kinds))], timeout=40)
         for cid, kind in enumerate(kinds):
             for r in range(n):
                 if kind == "reduce" and r != cid % n:
