@@ -254,6 +254,7 @@ struct Daemon {
     __atomic_store_n(ctrl, 0u, __ATOMIC_RELEASE);
     if (hipMemcpy(devArgs, &hostArgs, sizeof(hostArgs), hipMemcpyHostToDevice) != hipSuccess) return false;
     if (hipMemset(devFlags, 0, 64) != hipSuccess) return false;
+    if (hipStreamSynchronize(nullptr) != hipSuccess) return false;  // args and flags are in place before the launch
     if (dfcclLaunchDaemon(devArgs, nSlots, chans, stream) != hipSuccess) return false;
     if (hipEventRecord(doneEv, stream) != hipSuccess) return false;
     running = true;
@@ -296,6 +297,7 @@ struct Daemon {
     __atomic_store_n(ctrl, kCtrlQuitRequest, __ATOMIC_RELEASE);
     if (!cv.wait_for(lk, std::chrono::seconds(20), [&] { return !running; })) {
       fprintf(stderr, "dfccl: daemon did not leave on request, aborting it\n");
+      failed = true;  // the aborted kernel's state is abandoned: no relaunch
       __atomic_store_n(ctrl, kCtrlAbort, __ATOMIC_RELEASE);
       cv.wait_for(lk, std::chrono::seconds(20), [&] { return !running; });
     }
@@ -312,6 +314,7 @@ static void abortAllDaemonsAtExit() {
     Daemon* d = kv.second;
     std::unique_lock<std::mutex> lk(d->mu);
     if (d->running) {
+      d->failed = true;
       __atomic_store_n(d->ctrl, kCtrlAbort, __ATOMIC_RELEASE);
       d->cv.wait_for(lk, std::chrono::seconds(5), [&] { return !d->running; });
     }
@@ -361,6 +364,7 @@ static void destroyDaemon(Daemon* d) {
     if (d->running) {
       // every rank has left; whatever is still resident only has to notice
       if (!d->cv.wait_for(lk, std::chrono::seconds(10), [&] { return !d->running; })) {
+        d->failed = true;
         __atomic_store_n(d->ctrl, kCtrlAbort, __ATOMIC_RELEASE);
         d->cv.wait_for(lk, std::chrono::seconds(10), [&] { return !d->running; });
       }
@@ -485,6 +489,9 @@ static ncclResult_t allocGroupLocked(CommGroup* g) {
     HIPCHECK(hipMalloc((void**)&g->tileCtrs, (size_t)g->nRanks * 128));
     HIPCHECK(hipMemset(g->tileCtrs, 0, (size_t)g->nRanks * 128));
   }
+  // the daemon runs on a stream that does not synchronise with the null stream: the clears must have landed
+  // before it can look at this memory
+  HIPCHECK(hipStreamSynchronize(nullptr));
   return ncclSuccess;
 }
 
@@ -593,6 +600,7 @@ static int sqWrite(ofcclRankCtx* c, uint64_t sendbuff, uint64_t recvbuff, uint32
 static ncclResult_t runColl(const void* sendbuff, void* recvbuff, int collId, CallbackFunc cb, void* cbArgs,
                             ofcclRankCtx_t c) {
   if (c == nullptr || !c->finalized) return ncclInvalidUsage;
+  if (c->daemon->failed) return ncclSystemError;  // the daemon could not be launched, or had to be aborted
   if (collId < 0 || collId >= kMaxColls || c->collIndex[collId] < 0) return ncclInvalidArgument;
   if (((uint64_t)(uintptr_t)sendbuff & ~kPtrMask) || ((uint64_t)(uintptr_t)recvbuff & ~kPtrMask))
     return ncclInvalidArgument;
@@ -854,6 +862,7 @@ DFCCL_API ncclResult_t ofcclFinalizeRankCtx7StartHostThrds(ofcclRankCtx_t c) {
   HIPCHECK(hipMemset(R.dyn, 0, (size_t)maxCh * nCollsAlloc * sizeof(DynCtx)));
   HIPCHECK(hipMalloc((void**)&R.saved, (size_t)maxCh * sizeof(WgSaved)));
   HIPCHECK(hipMemset(R.saved, 0, (size_t)maxCh * sizeof(WgSaved)));
+  HIPCHECK(hipStreamSynchronize(nullptr));  // see allocGroupLocked
 
   // attach to the device daemon; a resident kernel has to leave first so that
   // the next launch covers this rank's workgroups
@@ -922,6 +931,8 @@ DFCCL_API ncclResult_t ofcclDestroy(ofcclRankCtx_t c) {
       }
       if (std::chrono::steady_clock::now() > deadline) {
         fprintf(stderr, "dfccl: rank %d did not leave the daemon, aborting the daemon\n", c->rank);
+        // an aborted kernel abandons its scheduler state: it must never be launched again on top of it
+        d->failed = true;
         __atomic_store_n(d->ctrl, kCtrlAbort, __ATOMIC_RELEASE);
         d->cv.wait_for(lk, std::chrono::seconds(10), [&] { return !d->running; });
         d->slots[c->slot] = nullptr;

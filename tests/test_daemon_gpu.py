@@ -473,3 +473,31 @@ def test_other_collectives_disordered_submission(proto):
                 if kind == "reduce" and r != cid % n:
                     continue
                 assert np.array_equal(to_np(orc.F32, bufs[cid][1][r]), wants[cid][r]), (cid, kind, r)
+
+
+@pytest.mark.skip(reason="was part of a GPU run that lost its box before any output came back; kept out of the "
+                         "suite until the run can be repeated safely")
+@pytest.mark.parametrize("knobs", [{"BASE_CTX_SWITCH_THRESHOLD": "1", "NUM_TRY_TASKQ_HEAD": "1", "RECV_SUCCESS_FACTOR": "0"},
+                                   {"DFCCL_EXPRESS": "0"}, {"DFCCL_IDLE_POLL_ROUNDS": "0"}, {}])
+def test_small_all_reduce_repeated_express_and_fallbacks(knobs, monkeypatch):
+    # the same small collective over and over (its context stays resident, so wave 0 runs it on the spot); with a
+    # spin budget of one poll most of those attempts run out at one of the two waits and hand over to the
+    # scheduler, because the ranks are submitted one after the other from this thread
+    from dfccl_amd.ring import VirtualRing
+    for k, v in knobs.items():
+        monkeypatch.setenv(k, v)
+    n, count = 4, 2048
+    with VirtualRing(n) as ring:
+        ring.prepare(0, "all_reduce", count, orc.F32, orc.SUM)
+        ring.prepare(1, "all_reduce", 3 * count, orc.BF16, orc.MAX)
+        ring.finalize()
+        for rep in range(40):
+            cid = rep % 3 // 2  # 0, 0, 1, 0, 0, 1, ...: the resident context changes now and then
+            dtype, op, cnt = (orc.F32, orc.SUM, count) if cid == 0 else (orc.BF16, orc.MAX, 3 * count)
+            sends_np, sends, recvs = make_buffers("all_reduce", dtype, n, cnt, 3000 + rep)
+            want = orc.all_reduce(dtype, op, geom_of(ring, cid), sends_np)
+            ring.run(cid, sends, recvs, timeout=30)
+            for r in range(n):
+                assert np.array_equal(to_np(dtype, recvs[r]), want[r]), (rep, r)
+        stats = ring.stats()
+        assert stats["cqesWritten"] == 40 * n
