@@ -21,8 +21,12 @@
 //    collectives per wave instruction instead of loading and spinning on each;
 //  * two data protocols: the reference's FIFO ring (slices staged through HBM
 //    FIFOs between neighbours) and a direct protocol in which the virtual ranks,
-//    whose buffers share one HBM, read each other's buffers in place and keep
-//    the ring's per-chunk accumulation order;
+//    whose buffers share one HBM, read each other's send buffers and write each
+//    other's receive buffers in place, keeping the ring's accumulation order;
+//    its buffers are announced when a submission is ingested, so ranks never
+//    wait for each other before the data has moved;
+//  * an idle leader keeps several polls of the host ring in flight, and a small
+//    all-reduce whose context is resident is run by wave 0 on the spot;
 //  * completions go to a host-coherent ring with a device-side ticket, no
 //    compare-and-swap over PCIe;
 //  * the collective's plan and resumable position live in LDS while it runs.

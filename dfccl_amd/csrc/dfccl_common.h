@@ -128,8 +128,8 @@ struct alignas(16) CollPlan {
 struct alignas(128) DynCtx {
   uint64_t sendbuff;
   uint64_t recvbuff;
-  int64_t gridOffset;   // loop the workgroup is in
-  int32_t step;         // ring step inside the loop
+  int64_t gridOffset;   // FIFO: first element of the loop the workgroup is in; direct: position of the sweep
+  int32_t step;         // FIFO: ring step inside the loop; direct: 0 = sweep, 2 = only the final wait is left
   int32_t slice;        // FIFO: slice inside the step's chunk; direct: 1 once the instance is published
   uint64_t sendStep;    // FIFO: slices ever sent on the send link (persists across instances)
   uint64_t recvStep;    // FIFO: slices ever received on the receive link
