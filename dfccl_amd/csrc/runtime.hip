@@ -304,6 +304,25 @@ struct Daemon {
   }
 };
 
+// What the host knows about every attached rank, printed before a daemon is aborted (caller holds d->mu).
+static void dumpDaemonState(const Daemon* d) {
+  fprintf(stderr, "dfccl: daemon on device %d: launch %u, %s\n", d->device, d->epoch, d->running ? "resident" : "not resident");
+  for (int s = 0; s < kMaxRankSlots; s++) {
+    const ofcclRankCtx* c = d->slots[s];
+    if (c == nullptr) continue;
+    fprintf(stderr, "dfccl:   slot %d rank %d: %llu submitted, %llu completed, %d channels; exit words (launch:kind)", s,
+            c->rank, (unsigned long long)c->submitted.load(), (unsigned long long)c->completed.load(), c->nChannels);
+    for (int ch = 0; ch < c->nChannels; ch++) {
+      const uint32_t w = __atomic_load_n(&c->dev.wgExit[ch], __ATOMIC_ACQUIRE);
+      fprintf(stderr, " %u:%u", w >> 4, w & 0xf);
+    }
+    fprintf(stderr, "\n");
+    for (size_t i = 0; i < c->colls.size(); i++)
+      if (c->inflight[c->colls[i].collId].load() != 0)
+        fprintf(stderr, "dfccl:     collective %d in flight\n", c->colls[i].collId);
+  }
+}
+
 static std::mutex gDaemonMu;
 static std::map<int, Daemon*> gDaemons;
 static bool gAtexitRegistered = false;
@@ -931,6 +950,7 @@ DFCCL_API ncclResult_t ofcclDestroy(ofcclRankCtx_t c) {
       }
       if (std::chrono::steady_clock::now() > deadline) {
         fprintf(stderr, "dfccl: rank %d did not leave the daemon, aborting the daemon\n", c->rank);
+        dumpDaemonState(d);
         // an aborted kernel abandons its scheduler state: it must never be launched again on top of it
         d->failed = true;
         __atomic_store_n(d->ctrl, kCtrlAbort, __ATOMIC_RELEASE);

@@ -73,7 +73,13 @@ class VirtualRing:
         for key in keys:
             left = deadline - time.monotonic()
             if left <= 0 or not self.done[key].wait(left):
-                raise TimeoutError(f"collective {key[1]} on rank {key[0]} did not complete within {timeout}s")
+                missing = [k for k in keys if not self.done[k].is_set()]
+                try:
+                    stats = self.stats()
+                except Exception as e:  # the counters are a diagnosis aid only
+                    stats = repr(e)
+                raise TimeoutError(f"collective {key[1]} on rank {key[0]} did not complete within {timeout}s; "
+                                   f"(rank, collective) still waited for: {missing}; daemon counters: {stats}")
 
     def stats(self):
         total = {}
