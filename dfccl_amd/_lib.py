@@ -56,6 +56,7 @@ SIGNATURES = {
     "ofcclRunAllGather": (_int, [_vp, _vp, _int, CALLBACK, _vp, _vp]),
     "dfcclReduceCopy": (_int, [ctypes.POINTER(_vp), _int, _vp, _sz, _int, _int, _sz, _vp]),
     "dfcclGetStats": (_int, [_vp, ctypes.POINTER(Stats)]),
+    "dfcclDumpState": (_int, [_vp]),
     "dfcclGetCollTiming": (_int, [_vp, _int, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64)]),
     "dfcclGetCollGeometry": (_int, [_vp, _int, ctypes.POINTER(CollGeometry)]),
 }

@@ -165,6 +165,10 @@ class RankCtx:
         self._run("ofcclRunBcast", coll_id, callback, buf)
 
     # -- introspection --------------------------------------------------------
+    def dump_state(self):
+        """What the host knows about the daemon, printed to stderr (a diagnosis aid when a collective hangs)."""
+        check(self.lib.dfcclDumpState(self.handle), "dfcclDumpState")
+
     def stats(self):
         s = Stats()
         check(self.lib.dfcclGetStats(self.handle, ctypes.byref(s)), "dfcclGetStats")

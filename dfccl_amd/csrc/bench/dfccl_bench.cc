@@ -204,6 +204,7 @@ struct World {
   }
   // what the daemon has done so far, rank by rank (printed when a run is given up)
   void report() {
+    (void)dfcclDumpState(ctx[0]);
     for (int r = 0; r < n; r++) {
       dfcclStats s{};
       if (dfcclGetStats(ctx[r], &s) != ncclSuccess) continue;

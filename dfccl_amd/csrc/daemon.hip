@@ -174,6 +174,31 @@ __device__ __forceinline__ void flushStats(const RankDev& R, WgShared& sh, int c
   __hip_atomic_store(&out->epoch, (uint64_t)epoch, __ATOMIC_RELEASE, DFCCL_SYSTEM);
 }
 
+// One thread: what the head of the task queue is parked on, for the host's diagnosis (see WgStats::stuck).
+__device__ __forceinline__ void reportStuck(const RankDev& R, WgShared& sh, int ch) {
+  DFCCL_GLOBAL WgStats* out = G(&R.stats[ch]);
+  const uint32_t coll = sh.taskq[0];
+  if (coll >= (uint32_t)R.nColls) return;
+  DynCtx d;
+  if ((int32_t)coll == sh.loadedColl) d = sh.dyn;
+  else loadStruct(d, &R.dyn[(size_t)ch * R.nColls + coll]);
+  uint64_t seen = 0;
+  if ((d.wait[0].count & (kWaitTagged - 1)) > 0)
+    seen = __hip_atomic_load((const DFCCL_GLOBAL uint64_t*)(uintptr_t)d.wait[0].ptr, __ATOMIC_RELAXED, DFCCL_AGENT);
+  const uint64_t n = __hip_atomic_load(&out->stuck[0], __ATOMIC_RELAXED, DFCCL_SYSTEM);
+  __hip_atomic_store(&out->stuck[1],
+                     (uint64_t)coll | ((uint64_t)(uint8_t)d.step << 32) | ((uint64_t)(uint8_t)d.slice << 40) |
+                         ((uint64_t)(uint16_t)sh.numActive << 48),
+                     __ATOMIC_RELAXED, DFCCL_SYSTEM);
+  __hip_atomic_store(&out->stuck[2], d.instance, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+  __hip_atomic_store(&out->stuck[3], d.wait[0].ptr, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+  __hip_atomic_store(&out->stuck[4], (d.wait[0].value & 0xffffffffffffull) | ((uint64_t)(uint16_t)d.wait[0].count << 48),
+                     __ATOMIC_RELAXED, DFCCL_SYSTEM);
+  __hip_atomic_store(&out->stuck[5], seen, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+  __hip_atomic_store(&out->stuck[6], d.wait[1].ptr, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+  __hip_atomic_store(&out->stuck[0], n + 1, __ATOMIC_RELEASE, DFCCL_SYSTEM);
+}
+
 // Wave 0: append the entries held one per lane (lanes < avail) to the task queue if this channel takes part
 // in them; a quit entry ends the batch.  (Role of checkSQ7TidyTaskQ, enqueue_ofccl_dev.cu:491-627.)
 __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane,
@@ -1241,6 +1266,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
         }
         if (sh.ingested > 0 || sh.progressedRound) sh.idle = 0;
         else sh.idle++;
+        if (sh.numActive > 0 && sh.idle > 0 && (sh.idle & (kStuckReportRounds - 1)) == 0) reportStuck(R, sh, ch);
         if (abortFlag) sh.exitKind = kExitAbort;
         else if (sh.finalQuit) sh.exitKind = kExitFinal;
         else if (quitFlag || expired) sh.exitKind = kExitVoluntary;

@@ -147,8 +147,14 @@ struct alignas(128) DynCtx {
 struct alignas(128) WgStats {
   uint64_t sqesRead, cqesWritten, ctxSaves, ctxLoads, voluntaryQuits, forcedQuits, slicesMoved, spins;
   uint64_t epoch;
-  uint64_t pad[7];
+  // Written by a workgroup that has had collectives queued without any progress for a long time (what the head
+  // of its task queue is parked on), for the host to print when it gives up on a daemon:
+  //   [0] reports so far  [1] collective index | step << 32 | published << 40 | queue length << 48
+  //   [2] instance  [3] first wait: address  [4] value waited for | count << 48  [5] value seen at that address
+  //   [6] second wait: address
+  uint64_t stuck[7];
 };
+constexpr int64_t kStuckReportRounds = 1 << 18;  // idle rounds between two such reports
 
 // Scheduler state a workgroup saves when it leaves voluntarily and restores at
 // the next launch (HBM).

@@ -319,7 +319,18 @@ static void dumpDaemonState(const Daemon* d) {
     fprintf(stderr, "\n");
     for (size_t i = 0; i < c->colls.size(); i++)
       if (c->inflight[c->colls[i].collId].load() != 0)
-        fprintf(stderr, "dfccl:     collective %d in flight\n", c->colls[i].collId);
+        fprintf(stderr, "dfccl:     collective %d (index %zu) in flight\n", c->colls[i].collId, i);
+    for (int ch = 0; ch < c->nChannels; ch++) {
+      const WgStats* st = &c->dev.stats[ch];
+      if (__atomic_load_n(&st->stuck[0], __ATOMIC_ACQUIRE) == 0) continue;
+      const uint64_t w1 = st->stuck[1], w4 = st->stuck[4];
+      fprintf(stderr, "dfccl:     channel %d parked %llu times: queue of %u headed by collective index %u, phase %u, "
+              "published %u, instance %llu; waits at %#llx for %llu (x%u), sees %#llx; second wait at %#llx\n", ch,
+              (unsigned long long)st->stuck[0], (unsigned)(w1 >> 48), (unsigned)(w1 & 0xffffffffu),
+              (unsigned)((w1 >> 32) & 0xff), (unsigned)((w1 >> 40) & 0xff), (unsigned long long)st->stuck[2],
+              (unsigned long long)st->stuck[3], (unsigned long long)(w4 & 0xffffffffffffull), (unsigned)(w4 >> 48),
+              (unsigned long long)st->stuck[5], (unsigned long long)st->stuck[6]);
+    }
   }
 }
 
@@ -1061,6 +1072,13 @@ DFCCL_API ncclResult_t dfcclGetStats(ofcclRankCtx_t c, dfcclStats* out) {
   }
   std::lock_guard<std::mutex> lk(d->mu);
   out->daemonLaunches = d->launches;
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t dfcclDumpState(ofcclRankCtx_t c) {
+  if (c == nullptr || !c->finalized) return ncclInvalidUsage;
+  std::lock_guard<std::mutex> lk(c->daemon->mu);
+  dumpDaemonState(c->daemon);
   return ncclSuccess;
 }
 

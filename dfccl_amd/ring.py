@@ -76,6 +76,7 @@ class VirtualRing:
                 missing = [k for k in keys if not self.done[k].is_set()]
                 try:
                     stats = self.stats()
+                    self.ctxs[0].dump_state()
                 except Exception as e:  # the counters are a diagnosis aid only
                     stats = repr(e)
                 raise TimeoutError(f"collective {key[1]} on rank {key[0]} did not complete within {timeout}s; "

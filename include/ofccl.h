@@ -192,6 +192,12 @@ typedef struct {
 } dfcclCollGeometry;
 ncclResult_t dfcclGetCollGeometry(ofcclRankCtx_t rankCtx, int collId, dfcclCollGeometry* geom);
 
+/* Prints to stderr what the host knows about the daemon this rank context is attached to: per rank the entries
+ * submitted and completed, how every workgroup left the last launch, the collectives in flight, and what a
+ * workgroup that has made no progress for a long time is parked on. (The reference prints comparable state under
+ * its DEBUG_* switches, src/collectives_ofccl/device/enqueue_ofccl_dev.cu:1290-1483.) */
+ncclResult_t dfcclDumpState(ofcclRankCtx_t rankCtx);
+
 #ifdef __cplusplus
 }
 #endif
