@@ -475,10 +475,13 @@ def test_other_collectives_disordered_submission(proto):
                 assert np.array_equal(to_np(orc.F32, bufs[cid][1][r]), wants[cid][r]), (cid, kind, r)
 
 
-@pytest.mark.skip(reason="was part of a GPU run that lost its box before any output came back; kept out of the "
-                         "suite until the run can be repeated safely")
-@pytest.mark.parametrize("knobs", [{"BASE_CTX_SWITCH_THRESHOLD": "1", "NUM_TRY_TASKQ_HEAD": "1", "RECV_SUCCESS_FACTOR": "0"},
-                                   {"DFCCL_EXPRESS": "0"}, {"DFCCL_IDLE_POLL_ROUNDS": "0"}, {}])
+@pytest.mark.skipif(os.environ.get("DFCCL_RUN_PARKED") != "1",
+                    reason="both GPU runs that included this test lost their box before any output came back and the "
+                           "cause is not known: not to be run on a GPU until it is (DFCCL_RUN_PARKED=1 runs it)")
+@pytest.mark.parametrize("knobs", [{"DFCCL_EXPRESS": "1", "BASE_CTX_SWITCH_THRESHOLD": "1", "NUM_TRY_TASKQ_HEAD": "1",
+                                    "RECV_SUCCESS_FACTOR": "0"},
+                                   {"DFCCL_EXPRESS": "0"}, {"DFCCL_EXPRESS": "1", "DFCCL_IDLE_POLL_ROUNDS": "0"},
+                                   {"DFCCL_EXPRESS": "1"}])
 def test_small_all_reduce_repeated_express_and_fallbacks(knobs, monkeypatch):
     # the same small collective over and over (its context stays resident, so wave 0 runs it on the spot); with a
     # spin budget of one poll most of those attempts run out at one of the two waits and hand over to the
