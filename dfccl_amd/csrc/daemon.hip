@@ -98,6 +98,23 @@ struct WgShared {
   uint8_t collChannels[kMaxColls];  // channels of every collective of this rank (copied from the plans at launch)
 };
 
+// the workgroup's one LDS object (a host build that emulates workgroups with threads supplies its own definition)
+#ifndef DFCCL_WG_SHARED
+#define DFCCL_WG_SHARED(T, name) __shared__ T name
+#endif
+
+// Marks the places where the lanes of one wave hand values to each other through LDS (one lane writes, the
+// others read afterwards, or the other way round).  The lanes of a wave run in lockstep, so on the GPU this is
+// nothing; a host build that runs every lane as a thread makes it a barrier of the wave.
+#ifndef DFCCL_WAVE_LDS_SYNC
+#define DFCCL_WAVE_LDS_SYNC()
+#endif
+// A value every lane of the wave loads from the same address with one instruction, and so gets identically;
+// lanes that run as threads of their own take lane 0's.
+#ifndef DFCCL_WAVE_UNIFORM
+#define DFCCL_WAVE_UNIFORM(x) (x)
+#endif
+
 #define DFCCL_AGENT __HIP_MEMORY_SCOPE_AGENT
 #define DFCCL_SYSTEM __HIP_MEMORY_SCOPE_SYSTEM
 
@@ -275,6 +292,7 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
     if (R.nChannels > 1) __hip_atomic_store(G(&R.wgFrontier[ch]), sh.frontier, __ATOMIC_RELAXED, DFCCL_AGENT);
     trace(A, sh, kTrIngested, (uint32_t)consumed);
   }
+  DFCCL_WAVE_LDS_SYNC();
 }
 
 // Leader, wave 0: fetch submissions from the host ring (four lanes per entry, each word validated by its own
@@ -292,7 +310,8 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
   const int idleRounds = (int)A.knobs.idlePollRounds;
   bool busy = false;
   if (sh.numActive == 0 && R.nChannels > 1)
-    busy = __hip_atomic_load(G(R.cqTicket), __ATOMIC_RELAXED, DFCCL_AGENT) < base;
+    busy = DFCCL_WAVE_UNIFORM(__hip_atomic_load(G(R.cqTicket), __ATOMIC_RELAXED, DFCCL_AGENT)) < base;
+  DFCCL_WAVE_LDS_SYNC();  // (every lane has read the state above)
   if (lane == 0) sh.rankBusy = busy ? 1 : 0;
   const bool idleMode = sh.numActive == 0 && idleRounds > 0 && !busy;
   const int nlanes = idleMode ? kSqeWords : kSqesPerPoll * kSqeWords;
@@ -354,6 +373,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
   while (n < kSqesPerPoll && ((vm >> (4 * n)) & 0xfull) == 0xfull) n++;
   if (n == 0) {
     if (lane == 0) sh.ingested = 0;
+    DFCCL_WAVE_LDS_SYNC();
   } else {
     // lane k < n takes entry k
     const int srcLane = (lane * 4) & 63;
@@ -380,6 +400,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
       sh.hostFrontier = base + (uint64_t)n;
       trace(A, sh, kTrSqeFetched, (uint32_t)n);
     }
+    DFCCL_WAVE_LDS_SYNC();
     ingestEntries(A, R, sh, 0, lane, n, sendbuff, recvbuff, coll, flags);
   }
   // The host may reuse entries every workgroup of the rank has consumed. It only looks at the head when the
@@ -391,10 +412,12 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
       if (lane < R.nChannels) f = __hip_atomic_load(G(&R.wgFrontier[lane]), __ATOMIC_RELAXED, DFCCL_AGENT);
       f = waveMin64(f);
     }
+    DFCCL_WAVE_LDS_SYNC();
     if (lane == 0 && f != sh.publishedHead) {
       __hip_atomic_store(G(R.sqHead), f, __ATOMIC_RELAXED, DFCCL_SYSTEM);
       sh.publishedHead = f;
     }
+    DFCCL_WAVE_LDS_SYNC();
   }
 }
 
@@ -402,10 +425,11 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
 __device__ __forceinline__ void ingestMirror(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane) {
   const uint64_t f = sh.frontier;
   // polled with a relaxed load: an acquire would invalidate the L2 on every poll of every idle workgroup
-  const uint64_t tail = __hip_atomic_load(G(R.mirrorTail), __ATOMIC_RELAXED, DFCCL_AGENT);
+  const uint64_t tail = DFCCL_WAVE_UNIFORM(__hip_atomic_load(G(R.mirrorTail), __ATOMIC_RELAXED, DFCCL_AGENT));
   const int avail = (int)((tail - f) < 64 ? (tail - f) : 64);
   if (avail <= 0) {
     if (lane == 0) sh.ingested = 0;
+    DFCCL_WAVE_LDS_SYNC();
     return;
   }
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -439,6 +463,7 @@ __device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, int ch
       sh.ready[0] = (n >= 64) ? ~0ull : ((1ull << n) - 1ull);
       sh.numReady = n;
     }
+    DFCCL_WAVE_LDS_SYNC();
     return;
   }
   for (int base = 0; base < n; base += 64) {
@@ -456,6 +481,7 @@ __device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, int ch
     total += __builtin_popcountll(m);
   }
   if (lane == 0) sh.numReady = total;
+  DFCCL_WAVE_LDS_SYNC();
 }
 
 // Wave 0: wait until both conditions hold.  Lanes 0..31 watch the counters of
@@ -467,6 +493,7 @@ __device__ __forceinline__ uint64_t waitDescs(const DaemonArgs& A, WgShared& sh,
   bool ok;
   int64_t spins = 0;
   uint64_t seen = 0;
+  DFCCL_WAVE_LDS_SYNC();  // (what thread 0 wrote before the call is read by every lane below)
   if (lane == 0) trace(A, sh, kTrWaitBegin, (uint32_t)((w0.count + w1.count) & 0xffff));
   const int64_t forceEvery = A.knobs.forceQuitEvery;
   if (forceEvery > 0 && sh.slicesSinceLoad >= forceEvery) {
@@ -506,6 +533,7 @@ __device__ __forceinline__ uint64_t waitDescs(const DaemonArgs& A, WgShared& sh,
       sh.dyn.wait[1] = w1;
     }
   }
+  DFCCL_WAVE_LDS_SYNC();
   return seen;
 }
 
@@ -879,6 +907,7 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
           if (lane < 32) sh.peerSend[lane] = word & kPtrMask;
           else sh.peerRecv[lane & 31] = word & kPtrMask;
         }
+        DFCCL_WAVE_LDS_SYNC();
         if (sh.waitOk && lane == 0) {
           SweepGeom& g = sh.sweep;
           const int kind = P.kind, root = P.root;
@@ -1068,6 +1097,7 @@ __device__ __forceinline__ bool runExpress(const DaemonArgs& A, const RankDev& R
     sh.slicesSinceLoad = 0;
     trace(A, sh, kTrVisitBegin, coll);
   }
+  DFCCL_WAVE_LDS_SYNC();
   // lanes 0..n-1 get the peers' send buffers, lanes 32..32+n-1 their receive buffers
   const WaitDesc w0 = waitFor(&P.pubs[0].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
   const WaitDesc w1 = waitFor(&P.pubs[0].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
@@ -1120,6 +1150,7 @@ __device__ __forceinline__ bool runExpress(const DaemonArgs& A, const RankDev& R
     sh.progressedRound = 1;
     sh.stats.slicesMoved++;
   }
+  DFCCL_WAVE_LDS_SYNC();
   const WaitDesc wp = waitFor(&P.p1[0], inst + 1, 8, n);
   waitDescs(A, sh, lane, wp, noWait(), false);
   if (!sh.waitOk) {
@@ -1130,6 +1161,7 @@ __device__ __forceinline__ bool runExpress(const DaemonArgs& A, const RankDev& R
       sh.stats.ctxSaves++;
       storeStruct(&R.dyn[(size_t)ch * R.nColls + coll], sh.dyn);
     }
+    DFCCL_WAVE_LDS_SYNC();
     return false;
   }
   if (lane == 0) {
@@ -1139,6 +1171,7 @@ __device__ __forceinline__ bool runExpress(const DaemonArgs& A, const RankDev& R
     sh.numActive = 0;
     trace(A, sh, kTrVisitEnd, 0);
   }
+  DFCCL_WAVE_LDS_SYNC();
   return true;
 }
 
@@ -1189,7 +1222,7 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
 }
 
 extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const DaemonArgs* __restrict__ argsPtr) {
-  __shared__ WgShared sh;
+  DFCCL_WG_SHARED(WgShared, sh);
   const DaemonArgs& A = *argsPtr;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // Workgroups go to the XCDs round robin.  The channels of a rank are rotated by its slot, so that the
@@ -1249,6 +1282,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
       if (sh.ingested > 0 && sh.express) runExpress(A, R, sh, ch, lane);
       if (sh.numActive > 0) scanReady(R, sh, ch, lane);
       else if (lane == 0) sh.numReady = 0;
+      DFCCL_WAVE_LDS_SYNC();
       if (lane == 0) {
         // the host's requests and the lifetime limit are looked at every 8th round: nobody waits on them
         uint32_t abortFlag = 0, quitFlag = 0;
@@ -1273,6 +1307,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
         else if (sh.idle >= K.tolerantUnprogressedCnt) sh.exitKind = kExitVoluntary;
         sh.progressedRound = 0;
       }
+      DFCCL_WAVE_LDS_SYNC();
       if (sh.numReady == 0 && sh.ingested == 0) {
         // nothing can move: the leader's next poll is a PCIe round trip anyway, the others back off a little
         if (ch != 0) __builtin_amdgcn_s_sleep(20);

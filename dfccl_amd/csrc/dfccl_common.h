@@ -21,7 +21,10 @@ constexpr int kMaxColls = 2000;      // collIds and collectives per rank context
 constexpr int kSqCapacity = 2000;    // submissions that may be outstanding per rank (QLen)
 constexpr int kSqRing = 2048;        // ring size, a power of two >= kSqCapacity + 1
 constexpr int kCqRing = 4096;        // completions can never outnumber kMaxColls in flight
-constexpr int kWgThreads = 512;      // daemon workgroup: 8 wave64
+#ifndef DFCCL_WG_THREADS  // (a host build of the kernels for testing may use fewer waves)
+#define DFCCL_WG_THREADS 512
+#endif
+constexpr int kWgThreads = DFCCL_WG_THREADS;  // daemon workgroup: 8 wave64
 constexpr int kMaxRankSlots = 16;    // virtual ranks one device daemon serves
 constexpr int kMaxChannels = 64;     // workgroups per virtual rank
 constexpr int kAlignBytes = 1024;    // chunk rounding unit: one wave's 128-bit access

@@ -97,7 +97,9 @@ __device__ __forceinline__ u32x4 packOp(u32x4 a, u32x4 b) {
   return r;
 }
 
+#ifndef DFCCL_GLOBAL  // (a host build of the kernels for testing defines it empty)
 #define DFCCL_GLOBAL __attribute__((address_space(1)))
+#endif
 
 // One element held in the low bits of a word (upper bits zero). Operands are in global memory.
 template <int ES>

@@ -13,7 +13,7 @@
 
 #include <stdint.h>
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define DFCCL_HD __host__ __device__ inline
 #else
 #define DFCCL_HD inline

@@ -1,0 +1,265 @@
+// Scenarios for the host emulation of the daemon kernel (see hip/hip_runtime.h here), through the public C ABI.
+// Each scenario runs collectives between virtual ranks, checks every result against a host loop, and ends with an
+// orderly teardown; a workgroup out of step, a run that stops moving, a bad address (AddressSanitizer build) or a
+// data race in LDS (ThreadSanitizer build) ends the process with a report.
+//
+//   emul_stress repeat <ranks> <count> <reps> <colls>   the same small fp32 Sum all-reduces over and over, one
+//        after the other, every rank submitted in turn from this thread (the shape of the parked GPU test
+//        test_small_all_reduce_repeated_express_and_fallbacks); knobs come from the environment
+//   emul_stress mixed <ranks> <reps>    all five collectives side by side, int32, ranks submit in different orders
+//   emul_stress relaunch <ranks>        idle exit and relaunch, with and without a collective parked
+#include <hip/hip_runtime.h>
+#include <ofccl.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <chrono>
+#include <string>
+#include <thread>
+#include <vector>
+
+#define CHECK(call)                                                                   \
+  do {                                                                                \
+    ncclResult_t r_ = (call);                                                         \
+    if (r_ != ncclSuccess) {                                                          \
+      fprintf(stderr, "%s:%d: %s -> %s\n", __FILE__, __LINE__, #call, ncclGetErrorString(r_)); \
+      exit(2);                                                                        \
+    }                                                                                 \
+  } while (0)
+
+extern "C" void emulDumpThreads();
+
+struct Ring {
+  int n = 0;
+  std::vector<ofcclRankCtx_t> ctxs;
+  std::vector<std::vector<ncclComm_t>> comms;  // per collective
+  std::vector<std::atomic<int>> done;          // completions per (rank, collective)
+  int ncolls = 0;
+  explicit Ring(int n_) : n(n_), ctxs((size_t)n_) {
+    for (int r = 0; r < n; r++) CHECK(ofcclInitRankCtx(&ctxs[r], r));
+  }
+  std::vector<ncclComm_t>& newComms() {
+    ncclUniqueId id;
+    CHECK(ncclGetUniqueId(&id));
+    std::vector<ncclComm_t> c((size_t)n);
+    for (int r = 0; r < n; r++) CHECK(ncclCommInitRank(&c[r], n, id, r));
+    comms.push_back(c);
+    ncolls++;
+    return comms.back();
+  }
+  void finalize() {
+    done = std::vector<std::atomic<int>>((size_t)n * ncolls);
+    for (auto& d : done) d.store(0);
+    for (int r = 0; r < n; r++) CHECK(ofcclFinalizeRankCtx7StartHostThrds(ctxs[r]));
+  }
+  std::atomic<int>& flag(int r, int cid) { return done[(size_t)r * ncolls + cid]; }
+  static int cb(int, void* arg) {
+    ((std::atomic<int>*)arg)->fetch_add(1);
+    return 0;
+  }
+  void waitAll(const std::vector<int>& want, double timeoutS, const char* what) {
+    const auto t0 = std::chrono::steady_clock::now();
+    for (;;) {
+      bool all = true;
+      for (int r = 0; r < n; r++)
+        for (int c = 0; c < ncolls; c++) all = all && flag(r, c).load() >= want[(size_t)r * ncolls + c];
+      if (all) return;
+      if (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > timeoutS) {
+        fprintf(stderr, "emul_stress: %s: not complete after %.0f s\n", what, timeoutS);
+        for (int r = 0; r < n; r++)
+          for (int c = 0; c < ncolls; c++)
+            if (flag(r, c).load() < want[(size_t)r * ncolls + c])
+              fprintf(stderr, "  rank %d collective %d: %d of %d\n", r, c, flag(r, c).load(), want[(size_t)r * ncolls + c]);
+        dfcclDumpState(ctxs[0]);
+        emulDumpThreads();
+        exit(3);
+      }
+      usleep(1000);
+    }
+  }
+  void destroy() {
+    for (int r = 0; r < n; r++) CHECK(ofcclDestroy(ctxs[r]));
+    for (auto& c : comms)
+      for (int r = 0; r < n; r++) CHECK(ncclCommDestroy(c[r]));
+  }
+};
+
+template <typename T>
+static T* devAlloc(size_t count) {
+  void* p = nullptr;
+  if (hipMalloc(&p, count * sizeof(T) + 16) != hipSuccess) exit(4);
+  return (T*)p;
+}
+
+static int scenarioRepeat(int n, int count, int reps, int ncolls) {
+  Ring ring(n);
+  for (int c = 0; c < ncolls; c++) {
+    auto& comms = ring.newComms();
+    for (int r = 0; r < n; r++) CHECK(ofcclPrepareAllReduce((size_t)count, ncclFloat32, ncclSum, comms[r], c, ring.ctxs[r]));
+  }
+  ring.finalize();
+  std::vector<float*> send((size_t)n), recv((size_t)n);
+  for (int r = 0; r < n; r++) {
+    send[r] = devAlloc<float>((size_t)count);
+    recv[r] = devAlloc<float>((size_t)count);
+  }
+  std::vector<int> want((size_t)n * ncolls, 0);
+  for (int rep = 0; rep < reps; rep++) {
+    const int cid = rep % ncolls;
+    for (int r = 0; r < n; r++)
+      for (int i = 0; i < count; i++) {
+        send[r][i] = (float)((i * 7 + r * 13 + rep) % 64);  // small integers: the sum is exact in any order
+        recv[r][i] = -1.0f;
+      }
+    for (int r = 0; r < n; r++) {
+      want[(size_t)r * ncolls + cid]++;
+      CHECK(ofcclRunAllReduce(send[r], recv[r], cid, Ring::cb, &ring.flag(r, cid), ring.ctxs[r]));
+    }
+    ring.waitAll(want, 120.0, "repeat");
+    for (int r = 0; r < n; r++)
+      for (int i = 0; i < count; i++) {
+        float s = 0;
+        for (int q = 0; q < n; q++) s += (float)((i * 7 + q * 13 + rep) % 64);
+        if (recv[r][i] != s) {
+          fprintf(stderr, "emul_stress: repeat: rep %d rank %d element %d: %g, expected %g\n", rep, r, i, recv[r][i], s);
+          return 1;
+        }
+      }
+  }
+  dfcclStats st;
+  uint64_t saves = 0, cqes = 0;
+  for (int r = 0; r < n; r++) {
+    CHECK(dfcclGetStats(ring.ctxs[r], &st));
+    saves += st.ctxSaves;
+    cqes += st.cqesWritten;
+  }
+  ring.destroy();
+  printf("repeat: %d ranks x %d reps of %d elements ok, %llu completions, %llu context saves\n", n, reps, count,
+         (unsigned long long)cqes, (unsigned long long)saves);
+  return 0;
+}
+
+// all five collectives, int32 Sum, every rank submits them in its own order, `reps` times
+static int scenarioMixed(int n, int reps) {
+  const int count = 3000, root = n - 1;
+  Ring ring(n);
+  const char* names[5] = {"all_reduce", "reduce_scatter", "all_gather", "reduce", "broadcast"};
+  for (int c = 0; c < 5; c++) {
+    auto& comms = ring.newComms();
+    for (int r = 0; r < n; r++) {
+      switch (c) {
+        case 0: CHECK(ofcclPrepareAllReduce(count, ncclInt32, ncclSum, comms[r], c, ring.ctxs[r])); break;
+        case 1: CHECK(ofcclPrepareReduceScatter(count, ncclInt32, ncclSum, comms[r], c, ring.ctxs[r])); break;
+        case 2: CHECK(ofcclPrepareAllGather(count, ncclInt32, comms[r], c, ring.ctxs[r])); break;
+        case 3: CHECK(ofcclPrepareReduce(count, ncclInt32, ncclSum, root, comms[r], c, ring.ctxs[r])); break;
+        default: CHECK(ofcclPrepareBroadcast(count, ncclInt32, root, comms[r], c, ring.ctxs[r])); break;
+      }
+    }
+  }
+  ring.finalize();
+  auto sendLen = [&](int c) { return c == 1 ? count * n : count; };
+  auto recvLen = [&](int c) { return c == 2 ? count * n : count; };
+  std::vector<std::vector<int32_t*>> send(5), recv(5);
+  for (int c = 0; c < 5; c++)
+    for (int r = 0; r < n; r++) {
+      send[c].push_back(devAlloc<int32_t>((size_t)sendLen(c)));
+      recv[c].push_back(devAlloc<int32_t>((size_t)recvLen(c)));
+    }
+  auto val = [](int c, int r, int i, int rep) { return (int32_t)(i * 31 + r * 1009 + c * 77 + rep); };
+  std::vector<int> want((size_t)n * 5, 0);
+  for (int rep = 0; rep < reps; rep++) {
+    for (int c = 0; c < 5; c++)
+      for (int r = 0; r < n; r++) {
+        for (int i = 0; i < sendLen(c); i++) send[c][r][i] = val(c, r, i, rep);
+        for (int i = 0; i < recvLen(c); i++) recv[c][r][i] = -7;
+      }
+    for (int k = 0; k < 5; k++)
+      for (int r = 0; r < n; r++) {
+        const int c = (k * (r % 2 ? 3 : 1) + r) % 5;  // every rank in its own order
+        want[(size_t)r * 5 + c]++;
+        auto* f = &ring.flag(r, c);
+        switch (c) {
+          case 0: CHECK(ofcclRunAllReduce(send[c][r], recv[c][r], c, Ring::cb, f, ring.ctxs[r])); break;
+          case 1: CHECK(ofcclRunReduceScatter(send[c][r], recv[c][r], c, Ring::cb, f, ring.ctxs[r])); break;
+          case 2: CHECK(ofcclRunAllGather(send[c][r], recv[c][r], c, Ring::cb, f, ring.ctxs[r])); break;
+          case 3: CHECK(ofcclRunReduce(send[c][r], recv[c][r], c, Ring::cb, f, ring.ctxs[r])); break;
+          default: CHECK(ofcclRunBroadcast(send[c][r], recv[c][r], c, Ring::cb, f, ring.ctxs[r])); break;
+        }
+      }
+    ring.waitAll(want, 180.0, "mixed");
+    for (int c = 0; c < 5; c++)
+      for (int r = 0; r < n; r++) {
+        if (c == 3 && r != root) continue;
+        for (int i = 0; i < recvLen(c); i++) {
+          int32_t e = 0;
+          if (c == 0 || c == 3) for (int q = 0; q < n; q++) e += val(c, q, i, rep);
+          else if (c == 1) for (int q = 0; q < n; q++) e += val(c, q, r * count + i, rep);
+          else if (c == 2) e = val(c, i / count, i % count, rep);
+          else e = val(c, root, i, rep);
+          if (recv[c][r][i] != e) {
+            fprintf(stderr, "emul_stress: mixed: rep %d %s rank %d element %d: %d, expected %d\n", rep, names[c], r, i,
+                    recv[c][r][i], e);
+            return 1;
+          }
+        }
+      }
+  }
+  ring.destroy();
+  printf("mixed: %d ranks x %d reps of the five collectives ok\n", n, reps);
+  return 0;
+}
+
+// idle exit and relaunch: one collective, a pause long enough for the daemon to leave, the collective again; then
+// one rank submits and the others only after the daemon has left with the collective parked
+static int scenarioRelaunch(int n) {
+  const int count = 5000;
+  Ring ring(n);
+  auto& comms = ring.newComms();
+  for (int r = 0; r < n; r++) CHECK(ofcclPrepareAllReduce(count, ncclInt32, ncclSum, comms[r], 0, ring.ctxs[r]));
+  ring.finalize();
+  std::vector<int32_t*> send, recv;
+  for (int r = 0; r < n; r++) {
+    send.push_back(devAlloc<int32_t>(count));
+    recv.push_back(devAlloc<int32_t>(count));
+  }
+  std::vector<int> want((size_t)n, 0);
+  for (int round = 0; round < 3; round++) {
+    for (int r = 0; r < n; r++)
+      for (int i = 0; i < count; i++) {
+        send[r][i] = i + r * 100 + round;
+        recv[r][i] = -1;
+      }
+    for (int r = 0; r < n; r++) {
+      want[r]++;
+      CHECK(ofcclRunAllReduce(send[r], recv[r], 0, Ring::cb, &ring.flag(r, 0), ring.ctxs[r]));
+      if (round == 2 && r == 0) sleep(3);  // the others come after rank 0's workgroup has given up and left
+    }
+    ring.waitAll(want, 180.0, "relaunch");
+    for (int r = 0; r < n; r++)
+      for (int i = 0; i < count; i++) {
+        int32_t e = 0;
+        for (int q = 0; q < n; q++) e += i + q * 100 + round;
+        if (recv[r][i] != e) {
+          fprintf(stderr, "emul_stress: relaunch: round %d rank %d element %d: %d, expected %d\n", round, r, i, recv[r][i], e);
+          return 1;
+        }
+      }
+    if (round == 0) sleep(3);  // idle: every workgroup leaves
+  }
+  dfcclStats st;
+  CHECK(dfcclGetStats(ring.ctxs[0], &st));
+  ring.destroy();
+  printf("relaunch: ok, %llu daemon launches, %llu voluntary exits of rank 0\n", (unsigned long long)st.daemonLaunches,
+         (unsigned long long)st.voluntaryQuits);
+  return st.daemonLaunches >= 2 ? 0 : 1;
+}
+
+int main(int argc, char** argv) {
+  setvbuf(stdout, nullptr, _IOLBF, 0);
+  const std::string mode = argc > 1 ? argv[1] : "";
+  if (mode == "repeat" && argc == 6) return scenarioRepeat(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]));
+  if (mode == "mixed" && argc == 4) return scenarioMixed(atoi(argv[2]), atoi(argv[3]));
+  if (mode == "relaunch" && argc == 3) return scenarioRelaunch(atoi(argv[2]));
+  fprintf(stderr, "usage: emul_stress repeat <ranks> <count> <reps> <colls> | mixed <ranks> <reps> | relaunch <ranks>\n");
+  return 64;
+}

@@ -1,0 +1,62 @@
+"""The daemon kernel's own source, compiled for the host and run with one OS thread per GPU thread
+(tests/emul/): scheduling, preemption, both protocols and the relaunch path without a GPU.
+
+What these runs can show that the GPU suite cannot show safely: a workgroup whose threads meet at different
+__syncthreads() (reported with both source lines; on the GPU that is a hang), a run that stops moving (every
+thread's position is printed) and, in the sanitizer builds (make -C tests/emul SAN=thread|address), races on LDS
+and bad addresses.  Random delays after barriers (EMUL_JITTER) let waves drift apart as they do on the GPU."""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+EMUL = os.path.join(HERE, "emul")
+CLANG = "/opt/rocm/lib/llvm/bin/clang++"
+
+pytestmark = pytest.mark.skipif(not os.path.exists(CLANG) or shutil.which("make") is None,
+                                reason="needs the ROCm clang++ and make to build the host emulation")
+
+
+@pytest.fixture(scope="module")
+def stress():
+    r = subprocess.run(["make", "-C", EMUL, "SAN=none", "-j4"], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    return os.path.join(EMUL, "_build", "none", "emul_stress")
+
+
+TINY = {"BASE_CTX_SWITCH_THRESHOLD": "1", "NUM_TRY_TASKQ_HEAD": "1", "RECV_SUCCESS_FACTOR": "0"}
+
+SCENARIOS = [
+    # the same small all-reduces over and over, ranks submitted in turn: scheduler path, then wave 0's express
+    # path, then the express path with every bounded wait giving up after one look
+    ("repeat-default", {}, ["repeat", "4", "2048", "12", "2"]),
+    ("repeat-express", {"DFCCL_EXPRESS": "1"}, ["repeat", "4", "2048", "12", "2"]),
+    ("repeat-express-tiny-budget", dict(TINY, DFCCL_EXPRESS="1"), ["repeat", "4", "2048", "20", "2"]),
+    ("repeat-tiny-budget-ragged", TINY, ["repeat", "3", "5000", "6", "2"]),
+    ("repeat-8-ranks", {}, ["repeat", "8", "2048", "4", "1"]),
+    ("repeat-several-channels", {}, ["repeat", "2", "300000", "2", "1"]),
+    # all five collectives side by side, ranks submit in different orders
+    ("mixed-direct", {}, ["mixed", "4", "2"]),
+    ("mixed-direct-tiny-budget", TINY, ["mixed", "4", "2"]),
+    ("mixed-fifo", {"DFCCL_PROTO": "fifo"}, ["mixed", "3", "2"]),
+    ("mixed-fifo-tiny-budget", dict(TINY, DFCCL_PROTO="fifo"), ["mixed", "3", "2"]),
+    # forced preemption after every slice / tile
+    ("forced-direct", {"DFCCL_FORCE_QUIT_EVERY": "1"}, ["repeat", "2", "40000", "2", "1"]),
+    ("forced-fifo", {"DFCCL_FORCE_QUIT_EVERY": "2", "DFCCL_PROTO": "fifo"}, ["repeat", "3", "40000", "2", "1"]),
+    # idle exit and relaunch, also with a collective parked
+    ("relaunch", {"TOLERANT_UNPROGRESSED_CNT": "200"}, ["relaunch", "2"]),
+]
+
+
+@pytest.mark.parametrize("name,env,args", SCENARIOS, ids=[s[0] for s in SCENARIOS])
+def test_emulated_daemon(stress, name, env, args):
+    e = dict(os.environ)
+    for k in ("DFCCL_PROTO", "DFCCL_EXPRESS", "DFCCL_FORCE_QUIT_EVERY", "BASE_CTX_SWITCH_THRESHOLD"):
+        e.pop(k, None)
+    e.update(env)
+    e.update({"EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "30", "DFCCL_DAEMON_MAX_MS": "100000"})
+    r = subprocess.run([stress] + args, env=e, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, f"{name}: rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
+    assert " ok" in r.stdout
