@@ -91,40 +91,75 @@ static T* devAlloc(size_t count) {
   return (T*)p;
 }
 
+static uint16_t bf16Of(int v) {  // small integers are exact in bfloat16
+  const float f = (float)v;
+  return (uint16_t)(__builtin_bit_cast(uint32_t, f) >> 16);
+}
+
+// Collective 0 is an fp32 Sum of `count` elements; a second one, if asked for, a bf16 Max of 3 * count.  With two
+// the order is 0, 0, 1, 0, 0, 1, ...: the context that is resident in the workgroup changes now and then, and
+// every second run of collective 0 finds its context resident (the condition of the express path).
 static int scenarioRepeat(int n, int count, int reps, int ncolls) {
   Ring ring(n);
+  if (ncolls > 2) ncolls = 2;
   for (int c = 0; c < ncolls; c++) {
     auto& comms = ring.newComms();
-    for (int r = 0; r < n; r++) CHECK(ofcclPrepareAllReduce((size_t)count, ncclFloat32, ncclSum, comms[r], c, ring.ctxs[r]));
+    for (int r = 0; r < n; r++) {
+      if (c == 0) CHECK(ofcclPrepareAllReduce((size_t)count, ncclFloat32, ncclSum, comms[r], c, ring.ctxs[r]));
+      else CHECK(ofcclPrepareAllReduce((size_t)count * 3, ncclBfloat16, ncclMax, comms[r], c, ring.ctxs[r]));
+    }
   }
   ring.finalize();
   std::vector<float*> send((size_t)n), recv((size_t)n);
+  std::vector<uint16_t*> sendB((size_t)n), recvB((size_t)n);
   for (int r = 0; r < n; r++) {
     send[r] = devAlloc<float>((size_t)count);
     recv[r] = devAlloc<float>((size_t)count);
+    sendB[r] = devAlloc<uint16_t>((size_t)count * 3);
+    recvB[r] = devAlloc<uint16_t>((size_t)count * 3);
   }
   std::vector<int> want((size_t)n * ncolls, 0);
   for (int rep = 0; rep < reps; rep++) {
-    const int cid = rep % ncolls;
-    for (int r = 0; r < n; r++)
+    const int cid = ncolls == 2 ? rep % 3 / 2 : 0;
+    auto valB = [&](int r, int i) { return (i * 5 + r * 37 + rep * 3) % 200 - 100; };
+    for (int r = 0; r < n; r++) {
       for (int i = 0; i < count; i++) {
         send[r][i] = (float)((i * 7 + r * 13 + rep) % 64);  // small integers: the sum is exact in any order
         recv[r][i] = -1.0f;
       }
+      for (int i = 0; i < count * 3; i++) {
+        sendB[r][i] = bf16Of(valB(r, i));
+        recvB[r][i] = 0x7fc0;
+      }
+    }
     for (int r = 0; r < n; r++) {
       want[(size_t)r * ncolls + cid]++;
-      CHECK(ofcclRunAllReduce(send[r], recv[r], cid, Ring::cb, &ring.flag(r, cid), ring.ctxs[r]));
+      if (cid == 0) CHECK(ofcclRunAllReduce(send[r], recv[r], cid, Ring::cb, &ring.flag(r, cid), ring.ctxs[r]));
+      else CHECK(ofcclRunAllReduce(sendB[r], recvB[r], cid, Ring::cb, &ring.flag(r, cid), ring.ctxs[r]));
     }
     ring.waitAll(want, 120.0, "repeat");
-    for (int r = 0; r < n; r++)
-      for (int i = 0; i < count; i++) {
-        float s = 0;
-        for (int q = 0; q < n; q++) s += (float)((i * 7 + q * 13 + rep) % 64);
-        if (recv[r][i] != s) {
-          fprintf(stderr, "emul_stress: repeat: rep %d rank %d element %d: %g, expected %g\n", rep, r, i, recv[r][i], s);
-          return 1;
+    for (int r = 0; r < n; r++) {
+      if (cid == 0) {
+        for (int i = 0; i < count; i++) {
+          float s = 0;
+          for (int q = 0; q < n; q++) s += (float)((i * 7 + q * 13 + rep) % 64);
+          if (recv[r][i] != s) {
+            fprintf(stderr, "emul_stress: repeat: rep %d rank %d element %d: %g, expected %g\n", rep, r, i, recv[r][i], s);
+            return 1;
+          }
+        }
+      } else {
+        for (int i = 0; i < count * 3; i++) {
+          int m = valB(0, i);
+          for (int q = 1; q < n; q++) m = valB(q, i) > m ? valB(q, i) : m;
+          if (recvB[r][i] != bf16Of(m)) {
+            fprintf(stderr, "emul_stress: repeat: rep %d rank %d bf16 element %d: %04x, expected %04x\n", rep, r, i,
+                    recvB[r][i], bf16Of(m));
+            return 1;
+          }
         }
       }
+    }
   }
   dfcclStats st;
   uint64_t saves = 0, cqes = 0;
