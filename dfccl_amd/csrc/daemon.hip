@@ -394,6 +394,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
       }
       // every lane's entry is written before lane 0 publishes the new tail
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      DFCCL_WAVE_LDS_SYNC();  // (the wave's fence covers all its lanes' stores)
       if (lane == 0) __hip_atomic_store(G(R.mirrorTail), base + (uint64_t)n, __ATOMIC_RELAXED, DFCCL_AGENT);
     }
     if (lane == 0) {

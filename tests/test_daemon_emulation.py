@@ -60,3 +60,29 @@ def test_emulated_daemon(stress, name, env, args):
     r = subprocess.run([stress] + args, env=e, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, f"{name}: rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
     assert " ok" in r.stdout
+
+
+DRIVER = [
+    # the native driver of the timing workloads on the emulation: per-rank host threads submit in different
+    # orders (disorder) or in bursts (buckets); the driver checks every result itself
+    ("disorder", ["disorder", "--ranks", "4", "--colls", "16", "--min-bytes", "4096", "--max-bytes", "65536",
+                  "--timeout", "250"]),
+    ("buckets", ["buckets", "--ranks", "4", "--colls", "6", "--elems", "20000", "--dtype", "bf16", "--iters", "1",
+                 "--warmup", "0", "--timeout", "250"]),
+    ("latency-8-ranks", ["latency", "--ranks", "8", "--bytes", "4096", "--dtype", "fp16", "--iters", "3", "--warmup", "1",
+                         "--timeout", "250"]),
+]
+
+
+@pytest.mark.parametrize("name,args", DRIVER, ids=[d[0] for d in DRIVER])
+def test_emulated_daemon_under_the_native_driver(stress, name, args):
+    import json
+    e = dict(os.environ)
+    e.update({"EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "60", "DFCCL_DAEMON_MAX_MS": "100000"})
+    exe = os.path.join(os.path.dirname(stress), "dfccl_bench_emul")
+    r = subprocess.run([exe] + args, env=e, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, f"{name}: rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert out["correct"] is True
+    if name == "disorder":
+        assert out["deadlocks"] == 0
