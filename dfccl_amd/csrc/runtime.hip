@@ -84,6 +84,9 @@ struct CommGroup {
   int handles = 0;
   // the collective this communicator serves, fixed by the first Prepare
   bool planned = false;
+  // a rank context that ran this collective has been destroyed: the counters in the group's device memory no
+  // longer match a fresh context's, so the communicator cannot be registered again
+  bool retired = false;
   int kind = 0, dtypeUser = 0, op = 0, root = 0;
   size_t countUser = 0;
   // derived plan
@@ -544,6 +547,7 @@ static ncclResult_t prepareColl(int kind, size_t count, int dtype, int op, int r
   {
     std::lock_guard<std::mutex> lk(g->mu);
     if (g->device != ctx->device) return ncclInvalidUsage;
+    if (g->retired) return ncclInvalidUsage;  // create a new communicator for a new rank context
     if (!g->planned) {
       g->kind = kind;
       g->dtypeUser = dtype;
@@ -998,7 +1002,13 @@ DFCCL_API ncclResult_t ofcclDestroy(ofcclRankCtx_t c) {
       }
     }
   }
-  for (auto& reg : c->colls) reg.comm->registered = false;
+  for (auto& reg : c->colls) {
+    reg.comm->registered = false;
+    if (c->finalized) {
+      std::lock_guard<std::mutex> lk(reg.comm->group->mu);
+      reg.comm->group->retired = true;
+    }
+  }
   if (c->device >= 0 && c->device < 64) gLiveRankCtxs[c->device].fetch_sub(1);
   delete c;
   return ncclSuccess;

@@ -105,7 +105,8 @@ ncclResult_t ofcclDestroy(ofcclRankCtx_t rankCtx);
 /* ---- prepare: register one collective under collId ------------------------
  * Validation follows src/enqueue_ofccl.cc:779-813 and src/misc/argcheck.cc:36-71:
  * collId in [0, 2000), at most 2000 collectives per context, a communicator
- * may be registered once, root / dtype / op in range.  Buffers are given at
+ * may be registered once (and not again after a rank context that ran its
+ * collective has been destroyed: create a new communicator), root / dtype / op in range.  Buffers are given at
  * Run time.  Unlike the reference (which drops `op` and always sums,
  * src/enqueue_ofccl.cc:211-215) Sum / Prod / Max / Min are honoured. */
 ncclResult_t ofcclPrepareReduce(size_t count, ncclDataType_t datatype, ncclRedOp_t op, int root, ncclComm_t comm,

@@ -8,6 +8,7 @@
 //        test_small_all_reduce_repeated_express_and_fallbacks); knobs come from the environment
 //   emul_stress mixed <ranks> <reps>    all five collectives side by side, int32, ranks submit in different orders
 //   emul_stress relaunch <ranks>        idle exit and relaunch, with and without a collective parked
+//   emul_stress reuse <ranks>           rank contexts destroyed and created again: old communicators are refused
 #include <hip/hip_runtime.h>
 #include <ofccl.h>
 #include <unistd.h>
@@ -289,12 +290,62 @@ static int scenarioRelaunch(int n) {
   return st.daemonLaunches >= 2 ? 0 : 1;
 }
 
+// A communicator whose collective has run cannot be registered with a new rank context (its device-side counters
+// would not match the fresh context's); a new communicator can, while the daemon of the first ring is still around.
+static int scenarioReuse(int n) {
+  const int count = 4000;
+  Ring ring(n);
+  auto comms = ring.newComms();
+  for (int r = 0; r < n; r++) CHECK(ofcclPrepareAllReduce(count, ncclInt32, ncclSum, comms[r], 0, ring.ctxs[r]));
+  ring.finalize();
+  std::vector<int32_t*> send, recv;
+  for (int r = 0; r < n; r++) {
+    send.push_back(devAlloc<int32_t>(count));
+    recv.push_back(devAlloc<int32_t>(count));
+    for (int i = 0; i < count; i++) send[r][i] = i + r;
+  }
+  std::vector<int> want((size_t)n, 1);
+  for (int r = 0; r < n; r++) CHECK(ofcclRunAllReduce(send[r], recv[r], 0, Ring::cb, &ring.flag(r, 0), ring.ctxs[r]));
+  ring.waitAll(want, 120.0, "reuse");
+  for (int r = 0; r < n; r++) CHECK(ofcclDestroy(ring.ctxs[r]));
+  // second generation of contexts
+  Ring ring2(n);
+  for (int r = 0; r < n; r++) {
+    const ncclResult_t res = ofcclPrepareAllReduce(count, ncclInt32, ncclSum, comms[r], 0, ring2.ctxs[r]);
+    if (res != ncclInvalidUsage) {
+      fprintf(stderr, "emul_stress: reuse: registering a used communicator returned %d\n", (int)res);
+      return 1;
+    }
+  }
+  auto& fresh = ring2.newComms();
+  for (int r = 0; r < n; r++) CHECK(ofcclPrepareAllReduce(count, ncclInt32, ncclSum, fresh[r], 0, ring2.ctxs[r]));
+  ring2.finalize();
+  for (int r = 0; r < n; r++)
+    for (int i = 0; i < count; i++) recv[r][i] = -1;
+  for (int r = 0; r < n; r++) CHECK(ofcclRunAllReduce(send[r], recv[r], 0, Ring::cb, &ring2.flag(r, 0), ring2.ctxs[r]));
+  ring2.waitAll(want, 120.0, "reuse, second generation");
+  for (int r = 0; r < n; r++)
+    for (int i = 0; i < count; i++) {
+      int32_t e = 0;
+      for (int q = 0; q < n; q++) e += i + q;
+      if (recv[r][i] != e) {
+        fprintf(stderr, "emul_stress: reuse: rank %d element %d: %d, expected %d\n", r, i, recv[r][i], e);
+        return 1;
+      }
+    }
+  ring2.destroy();
+  for (int r = 0; r < n; r++) CHECK(ncclCommDestroy(comms[r]));
+  printf("reuse: ok\n");
+  return 0;
+}
+
 int main(int argc, char** argv) {
   setvbuf(stdout, nullptr, _IOLBF, 0);
   const std::string mode = argc > 1 ? argv[1] : "";
   if (mode == "repeat" && argc == 6) return scenarioRepeat(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]));
   if (mode == "mixed" && argc == 4) return scenarioMixed(atoi(argv[2]), atoi(argv[3]));
   if (mode == "relaunch" && argc == 3) return scenarioRelaunch(atoi(argv[2]));
-  fprintf(stderr, "usage: emul_stress repeat <ranks> <count> <reps> <colls> | mixed <ranks> <reps> | relaunch <ranks>\n");
+  if (mode == "reuse" && argc == 3) return scenarioReuse(atoi(argv[2]));
+  fprintf(stderr, "usage: emul_stress repeat <ranks> <count> <reps> <colls> | mixed <ranks> <reps> | relaunch <ranks> | reuse <ranks>\n");
   return 64;
 }

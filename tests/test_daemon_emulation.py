@@ -47,6 +47,8 @@ SCENARIOS = [
     ("forced-fifo", {"DFCCL_FORCE_QUIT_EVERY": "2", "DFCCL_PROTO": "fifo"}, ["repeat", "3", "40000", "2", "1"]),
     # idle exit and relaunch, also with a collective parked
     ("relaunch", {"TOLERANT_UNPROGRESSED_CNT": "200"}, ["relaunch", "2"]),
+    # rank contexts destroyed and created again on the same daemon; a communicator that has run is refused
+    ("reuse", {}, ["reuse", "3"]),
 ]
 
 
