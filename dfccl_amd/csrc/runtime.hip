@@ -1058,7 +1058,8 @@ DFCCL_API ncclResult_t dfcclGetStats(ofcclRankCtx_t c, dfcclStats* out) {
       if (e == 0) e = ++d->statsEpoch;
       __atomic_store_n(&d->ctrl[1], e, __ATOMIC_RELEASE);
       lk.unlock();
-      const uint64_t deadline = nowNs() + 20000000ull;
+      // (20 ms is ample on the GPU; DFCCL_STATS_WAIT_MS is for hosts where the daemon runs much slower than that)
+      const uint64_t deadline = nowNs() + (uint64_t)envInt("DFCCL_STATS_WAIT_MS", 20) * 1000000ull;
       for (;;) {
         bool all = true;
         for (int ch = 0; ch < c->nChannels && all; ch++)

