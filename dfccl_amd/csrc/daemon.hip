@@ -104,10 +104,20 @@ struct WgShared {
 #endif
 
 // Marks the places where the lanes of one wave hand values to each other through LDS (one lane writes, the
-// others read afterwards, or the other way round).  The lanes of a wave run in lockstep, so on the GPU this is
-// nothing; a host build that runs every lane as a thread makes it a barrier of the wave.
+// others read afterwards, or the other way round).  The hardware runs the lanes of a wave in lockstep and its LDS
+// accesses in order, but the compiler knows nothing of that: to it the lanes are independent threads without
+// synchronisation, and it has been seen to place the other lanes' read of a flag before the branch in which
+// lane 0 writes it (so that lane 0 saw a failed wait and the other 63 lanes a successful one).  The barrier of
+// the wave is a convergent operation: every lane's earlier accesses stay before it and every later access after
+// it, and it is not moved into either side of a branch.  It costs no instruction.  (A host build that runs
+// every lane as a thread makes it a real barrier of the wave.)
 #ifndef DFCCL_WAVE_LDS_SYNC
-#define DFCCL_WAVE_LDS_SYNC()
+#define DFCCL_WAVE_LDS_SYNC()                               \
+  do {                                                      \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  \
+    __builtin_amdgcn_wave_barrier();                        \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");  \
+  } while (0)
 #endif
 // A value every lane of the wave loads from the same address with one instruction, and so gets identically;
 // lanes that run as threads of their own take lane 0's.
