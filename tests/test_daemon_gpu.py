@@ -478,8 +478,9 @@ def test_other_collectives_disordered_submission(proto):
 
 
 @pytest.mark.skipif(os.environ.get("DFCCL_RUN_PARKED") != "1",
-                    reason="both GPU runs that included this test lost their box before any output came back and the "
-                           "cause is not known: not to be run on a GPU until it is (DFCCL_RUN_PARKED=1 runs it)")
+                    reason="both GPU runs that included this test lost their box (a wave's lanes read a flag in LDS "
+                           "before lane 0 had written it; fixed since, passes on the host emulation); its one "
+                           "confirming run on a GPU is still to come (DFCCL_RUN_PARKED=1 runs it)")
 @pytest.mark.parametrize("knobs", [{"DFCCL_EXPRESS": "1", "BASE_CTX_SWITCH_THRESHOLD": "1", "NUM_TRY_TASKQ_HEAD": "1",
                                     "RECV_SUCCESS_FACTOR": "0"},
                                    {"DFCCL_EXPRESS": "0"}, {"DFCCL_EXPRESS": "1", "DFCCL_IDLE_POLL_ROUNDS": "0"},
