@@ -221,9 +221,8 @@ struct Daemon {
     knobs.tolerantUnprogressedCnt = envInt("TOLERANT_UNPROGRESSED_CNT", 500000);
     knobs.forceQuitEvery = envInt("DFCCL_FORCE_QUIT_EVERY", 0);
     knobs.maxLifetimeTicks = envInt("DFCCL_DAEMON_MAX_MS", 0) * 100000;  // wall_clock64 runs at 100 MHz
-    // Off unless asked for: a stress test of this path with a spin limit of 1 (every bounded wait gives up and
-    // hands over to the scheduler) faulted the GPU; the cause is fixed (see DFCCL_WAVE_LDS_SYNC in daemon.hip), the
-    // test has not been run on a GPU again yet.
+    // Off unless asked for: its stress test (spin limit 1, every bounded wait gives up) faulted the GPU; the cause
+    // is fixed (see DFCCL_WAVE_LDS_SYNC in daemon.hip) but the test has not been run on a GPU again yet.
     knobs.express = envInt("DFCCL_EXPRESS", 0);
     knobs.idlePollRounds = envInt("DFCCL_IDLE_POLL_ROUNDS", 8);
     if (knobs.numTryTaskqHead < 1) knobs.numTryTaskqHead = 1;
