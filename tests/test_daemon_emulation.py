@@ -47,6 +47,10 @@ SCENARIOS = [
     ("forced-fifo", {"DFCCL_FORCE_QUIT_EVERY": "2", "DFCCL_PROTO": "fifo"}, ["repeat", "3", "40000", "2", "1"]),
     # idle exit and relaunch, also with a collective parked
     ("relaunch", {"TOLERANT_UNPROGRESSED_CNT": "200"}, ["relaunch", "2"]),
+    # a daemon that leaves every 50 ms, whatever it is doing, and is launched again: state saved and restored
+    ("short-lifetime-direct", {"DFCCL_DAEMON_MAX_MS": "50"}, ["mixed", "4", "2"]),
+    ("short-lifetime-fifo", {"DFCCL_DAEMON_MAX_MS": "50", "DFCCL_PROTO": "fifo"}, ["mixed", "3", "2"]),
+    ("short-lifetime-express", {"DFCCL_DAEMON_MAX_MS": "50", "DFCCL_EXPRESS": "1"}, ["repeat", "4", "2048", "20", "2"]),
     # rank contexts destroyed and created again on the same daemon; a communicator that has run is refused
     ("reuse", {}, ["reuse", "3"]),
 ]
@@ -57,8 +61,8 @@ def test_emulated_daemon(stress, name, env, args):
     e = dict(os.environ)
     for k in ("DFCCL_PROTO", "DFCCL_EXPRESS", "DFCCL_FORCE_QUIT_EVERY", "BASE_CTX_SWITCH_THRESHOLD"):
         e.pop(k, None)
-    e.update(env)
     e.update({"EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "30", "DFCCL_DAEMON_MAX_MS": "100000"})
+    e.update(env)
     r = subprocess.run([stress] + args, env=e, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, f"{name}: rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
     assert " ok" in r.stdout
