@@ -9,6 +9,7 @@
 //   emul_stress mixed <ranks> <reps>    all five collectives side by side, int32, ranks submit in different orders
 //   emul_stress relaunch <ranks>        idle exit and relaunch, with and without a collective parked
 //   emul_stress reuse <ranks>           rank contexts destroyed and created again: old communicators are refused
+//   emul_stress fuzz <seed> <rounds>    random collectives, ranks and submission orders
 #include <hip/hip_runtime.h>
 #include <ofccl.h>
 #include <unistd.h>
@@ -339,6 +340,108 @@ static int scenarioReuse(int n) {
   return 0;
 }
 
+// Random collectives (kind, count, root), every rank submits them in its own random order, several rounds; int32
+// Sum so that any result can be checked exactly.  The knobs come from the environment.
+static int scenarioFuzz(uint64_t seed, int rounds) {
+  uint64_t x = seed * 0x9e3779b97f4a7c15ull + 12345;
+  auto rnd = [&](uint64_t m) {
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    return (x >> 11) % m;
+  };
+  const int n = 2 + (int)rnd(5), ncolls = 1 + (int)rnd(7);
+  struct Coll { int kind, count, root; };
+  std::vector<Coll> colls;
+  Ring ring(n);
+  for (int c = 0; c < ncolls; c++) {
+    Coll k;
+    k.kind = (int)rnd(5);
+    const int shape = (int)rnd(4);
+    k.count = shape == 0 ? 1 + (int)rnd(16) : shape == 1 ? 1 + (int)rnd(3000) : shape == 2 ? 256 * (1 + (int)rnd(40)) : 1 + (int)rnd(60000);
+    k.root = (int)rnd((uint64_t)n);
+    colls.push_back(k);
+    auto& comms = ring.newComms();
+    for (int r = 0; r < n; r++) {
+      switch (k.kind) {
+        case 0: CHECK(ofcclPrepareAllReduce(k.count, ncclInt32, ncclSum, comms[r], c, ring.ctxs[r])); break;
+        case 1: CHECK(ofcclPrepareReduceScatter(k.count, ncclInt32, ncclSum, comms[r], c, ring.ctxs[r])); break;
+        case 2: CHECK(ofcclPrepareAllGather(k.count, ncclInt32, comms[r], c, ring.ctxs[r])); break;
+        case 3: CHECK(ofcclPrepareReduce(k.count, ncclInt32, ncclSum, k.root, comms[r], c, ring.ctxs[r])); break;
+        default: CHECK(ofcclPrepareBroadcast(k.count, ncclInt32, k.root, comms[r], c, ring.ctxs[r])); break;
+      }
+    }
+  }
+  ring.finalize();
+  auto sendLen = [&](int c) { return colls[c].kind == 1 ? colls[c].count * n : colls[c].count; };
+  auto recvLen = [&](int c) { return colls[c].kind == 2 ? colls[c].count * n : colls[c].count; };
+  std::vector<std::vector<int32_t*>> send((size_t)ncolls), recv((size_t)ncolls);
+  for (int c = 0; c < ncolls; c++)
+    for (int r = 0; r < n; r++) {
+      send[c].push_back(devAlloc<int32_t>((size_t)sendLen(c)));
+      recv[c].push_back(devAlloc<int32_t>((size_t)recvLen(c)));
+    }
+  auto val = [](int c, int r, int i, int rep) { return (int32_t)(i * 31 + r * 1009 + c * 77 + rep * 5); };
+  std::vector<int> want((size_t)n * ncolls, 0);
+  for (int rep = 0; rep < rounds; rep++) {
+    for (int c = 0; c < ncolls; c++)
+      for (int r = 0; r < n; r++) {
+        for (int i = 0; i < sendLen(c); i++) send[c][r][i] = val(c, r, i, rep);
+        for (int i = 0; i < recvLen(c); i++) recv[c][r][i] = -7;
+      }
+    // per-rank random order; ranks are interleaved at random as well
+    std::vector<std::vector<int>> order((size_t)n);
+    for (int r = 0; r < n; r++) {
+      for (int c = 0; c < ncolls; c++) order[r].push_back(c);
+      for (int i = ncolls - 1; i > 0; i--) std::swap(order[r][i], order[r][rnd((uint64_t)i + 1)]);
+    }
+    std::vector<int> next((size_t)n, 0);
+    for (int left = n * ncolls; left > 0;) {
+      const int r = (int)rnd((uint64_t)n);
+      if (next[r] >= ncolls) continue;
+      const int c = order[r][next[r]++];
+      left--;
+      want[(size_t)r * ncolls + c]++;
+      auto* f = &ring.flag(r, c);
+      switch (colls[c].kind) {
+        case 0: CHECK(ofcclRunAllReduce(send[c][r], recv[c][r], c, Ring::cb, f, ring.ctxs[r])); break;
+        case 1: CHECK(ofcclRunReduceScatter(send[c][r], recv[c][r], c, Ring::cb, f, ring.ctxs[r])); break;
+        case 2: CHECK(ofcclRunAllGather(send[c][r], recv[c][r], c, Ring::cb, f, ring.ctxs[r])); break;
+        case 3: CHECK(ofcclRunReduce(send[c][r], recv[c][r], c, Ring::cb, f, ring.ctxs[r])); break;
+        default: CHECK(ofcclRunBroadcast(send[c][r], recv[c][r], c, Ring::cb, f, ring.ctxs[r])); break;
+      }
+      if (rnd(4) == 0) usleep((useconds_t)rnd(3000));
+    }
+    ring.waitAll(want, 240.0, "fuzz");
+    for (int c = 0; c < ncolls; c++)
+      for (int r = 0; r < n; r++) {
+        const int kind = colls[c].kind, count = colls[c].count, root = colls[c].root;
+        if (kind == 3 && r != root) continue;
+        for (int i = 0; i < recvLen(c); i++) {
+          int32_t e = 0;
+          if (kind == 0 || kind == 3) for (int q = 0; q < n; q++) e += val(c, q, i, rep);
+          else if (kind == 1) for (int q = 0; q < n; q++) e += val(c, q, r * count + i, rep);
+          else if (kind == 2) e = val(c, i / count, i % count, rep);
+          else e = val(c, root, i, rep);
+          if (recv[c][r][i] != e) {
+            fprintf(stderr, "emul_stress: fuzz seed %llu: round %d collective %d (kind %d, count %d, root %d) rank %d of %d "
+                    "element %d: %d, expected %d\n", (unsigned long long)seed, rep, c, kind, count, root, r, n, i,
+                    recv[c][r][i], e);
+            return 1;
+          }
+        }
+      }
+  }
+  ring.destroy();
+  for (int c = 0; c < ncolls; c++)
+    for (int r = 0; r < n; r++) {
+      hipFree(send[c][r]);
+      hipFree(recv[c][r]);
+    }
+  printf("fuzz: seed %llu: %d ranks, %d collectives, %d rounds ok\n", (unsigned long long)seed, n, ncolls, rounds);
+  return 0;
+}
+
 int main(int argc, char** argv) {
   setvbuf(stdout, nullptr, _IOLBF, 0);
   const std::string mode = argc > 1 ? argv[1] : "";
@@ -346,6 +449,7 @@ int main(int argc, char** argv) {
   if (mode == "mixed" && argc == 4) return scenarioMixed(atoi(argv[2]), atoi(argv[3]));
   if (mode == "relaunch" && argc == 3) return scenarioRelaunch(atoi(argv[2]));
   if (mode == "reuse" && argc == 3) return scenarioReuse(atoi(argv[2]));
-  fprintf(stderr, "usage: emul_stress repeat <ranks> <count> <reps> <colls> | mixed <ranks> <reps> | relaunch <ranks> | reuse <ranks>\n");
+  if (mode == "fuzz" && argc == 4) return scenarioFuzz(strtoull(argv[2], nullptr, 10), atoi(argv[3]));
+  fprintf(stderr, "usage: emul_stress repeat <ranks> <count> <reps> <colls> | mixed <ranks> <reps> | relaunch <ranks> | reuse <ranks> | fuzz <seed> <rounds>\n");
   return 64;
 }

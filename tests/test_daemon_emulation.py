@@ -51,6 +51,11 @@ SCENARIOS = [
     ("short-lifetime-direct", {"DFCCL_DAEMON_MAX_MS": "50"}, ["mixed", "4", "2"]),
     ("short-lifetime-fifo", {"DFCCL_DAEMON_MAX_MS": "50", "DFCCL_PROTO": "fifo"}, ["mixed", "3", "2"]),
     ("short-lifetime-express", {"DFCCL_DAEMON_MAX_MS": "50", "DFCCL_EXPRESS": "1"}, ["repeat", "4", "2048", "20", "2"]),
+    # random ranks, collectives, sizes, roots and submission orders (three rounds each)
+    ("random-direct", {"NCCL_MAX_NCHANNELS": "2"}, ["fuzz", "1003", "3"]),
+    ("random-fifo-short-lifetime", {"NCCL_MAX_NCHANNELS": "2", "DFCCL_PROTO": "fifo", "DFCCL_DAEMON_MAX_MS": "57"},
+     ["fuzz", "1007", "3"]),
+    ("random-express-tiny-budget", dict(TINY, NCCL_MAX_NCHANNELS="2", DFCCL_EXPRESS="1"), ["fuzz", "1012", "3"]),
     # rank contexts destroyed and created again on the same daemon; a communicator that has run is refused
     ("reuse", {}, ["reuse", "3"]),
 ]
