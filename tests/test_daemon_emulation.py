@@ -66,7 +66,7 @@ def test_emulated_daemon(stress, name, env, args):
     e = dict(os.environ)
     for k in ("DFCCL_PROTO", "DFCCL_EXPRESS", "DFCCL_FORCE_QUIT_EVERY", "BASE_CTX_SWITCH_THRESHOLD"):
         e.pop(k, None)
-    e.update({"EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "30", "DFCCL_DAEMON_MAX_MS": "100000"})
+    e.update({"EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "120", "DFCCL_DAEMON_MAX_MS": "100000"})
     e.update(env)
     r = subprocess.run([stress] + args, env=e, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, f"{name}: rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
@@ -89,7 +89,7 @@ DRIVER = [
 def test_emulated_daemon_under_the_native_driver(stress, name, args):
     import json
     e = dict(os.environ)
-    e.update({"EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "60", "DFCCL_DAEMON_MAX_MS": "100000"})
+    e.update({"EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "120", "DFCCL_DAEMON_MAX_MS": "100000"})
     exe = os.path.join(os.path.dirname(stress), "dfccl_bench_emul")
     r = subprocess.run([exe] + args, env=e, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, f"{name}: rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
@@ -108,7 +108,7 @@ def test_parity_tests_on_the_emulation(stress):
     import sys
     e = dict(os.environ)
     e.update({"DFCCL_TESTS_ON_EMULATION": os.path.join(os.path.dirname(stress), "libdfccl_emul.so"),
-              "EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "90"})
+              "EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "120"})
     pick = ("test_small_all_reduce_and_in_place or test_in_place_and_absent_buffers or golden or "
             "test_other_collectives_disordered or test_rank_by_rank or forced_preemption")
     r = subprocess.run([sys.executable, "-m", "pytest", os.path.join(HERE, "test_daemon_gpu.py"),
