@@ -86,11 +86,17 @@ struct Ring {
   }
 };
 
+static std::vector<void*> gBuffers;  // everything devAlloc handed out since the last freeBuffers()
 template <typename T>
 static T* devAlloc(size_t count) {
   void* p = nullptr;
   if (hipMalloc(&p, count * sizeof(T) + 16) != hipSuccess) exit(4);
+  gBuffers.push_back(p);
   return (T*)p;
+}
+static void freeBuffers() {
+  for (void* p : gBuffers) hipFree(p);
+  gBuffers.clear();
 }
 
 static uint16_t bf16Of(int v) {  // small integers are exact in bfloat16
@@ -171,6 +177,7 @@ static int scenarioRepeat(int n, int count, int reps, int ncolls) {
     cqes += st.cqesWritten;
   }
   ring.destroy();
+  freeBuffers();
   printf("repeat: %d ranks x %d reps of %d elements ok, %llu completions, %llu context saves\n", n, reps, count,
          (unsigned long long)cqes, (unsigned long long)saves);
   return 0;
@@ -242,6 +249,7 @@ static int scenarioMixed(int n, int reps) {
       }
   }
   ring.destroy();
+  freeBuffers();
   printf("mixed: %d ranks x %d reps of the five collectives ok\n", n, reps);
   return 0;
 }
@@ -286,6 +294,7 @@ static int scenarioRelaunch(int n) {
   dfcclStats st;
   CHECK(dfcclGetStats(ring.ctxs[0], &st));
   ring.destroy();
+  freeBuffers();
   printf("relaunch: ok, %llu daemon launches, %llu voluntary exits of rank 0\n", (unsigned long long)st.daemonLaunches,
          (unsigned long long)st.voluntaryQuits);
   return st.daemonLaunches >= 2 ? 0 : 1;
@@ -335,6 +344,7 @@ static int scenarioReuse(int n) {
       }
     }
   ring2.destroy();
+  freeBuffers();
   for (int r = 0; r < n; r++) CHECK(ncclCommDestroy(comms[r]));
   printf("reuse: ok\n");
   return 0;
@@ -433,17 +443,14 @@ static int scenarioFuzz(uint64_t seed, int rounds) {
       }
   }
   ring.destroy();
-  for (int c = 0; c < ncolls; c++)
-    for (int r = 0; r < n; r++) {
-      hipFree(send[c][r]);
-      hipFree(recv[c][r]);
-    }
+  freeBuffers();
   printf("fuzz: seed %llu: %d ranks, %d collectives, %d rounds ok\n", (unsigned long long)seed, n, ncolls, rounds);
   return 0;
 }
 
 int main(int argc, char** argv) {
   setvbuf(stdout, nullptr, _IOLBF, 0);
+  setenv("DFCCL_STATS_WAIT_MS", "5000", 0);  // emulated workgroups answer a request for their counters slowly
   const std::string mode = argc > 1 ? argv[1] : "";
   if (mode == "repeat" && argc == 6) return scenarioRepeat(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]));
   if (mode == "mixed" && argc == 4) return scenarioMixed(atoi(argv[2]), atoi(argv[3]));
