@@ -26,7 +26,8 @@
 //    its buffers are announced when a submission is ingested, so ranks never
 //    wait for each other before the data has moved;
 //  * an idle leader keeps several polls of the host ring in flight, and a small
-//    all-reduce whose context is resident is run by wave 0 on the spot;
+//    collective (one tile of a few KiB) is run by wave 0 alone, without a single
+//    workgroup barrier between its waits and its data movement;
 //  * completions go to a host-coherent ring with a device-side ticket, no
 //    compare-and-swap over PCIe;
 //  * the collective's plan and resumable position live in LDS while it runs.
@@ -40,7 +41,7 @@ namespace dfccl {
 constexpr int kDaemonUnroll = 1;  // see reduce_copy.hip: shallow unrolling keeps DRAM accesses ordered
 constexpr int kReadyWords = (kMaxColls + 63) / 64;
 constexpr int kSoftWaitSpins = 2;       // polls of a wait of the direct protocol while other collectives are queued
-constexpr int kExpressMaxBytes = 4096;  // largest own chunk wave 0 folds by itself (see runExpress)
+constexpr int kSoloMaxBytes = 4096;  // largest own chunk of a one-tile collective that wave 0 runs by itself (see runDirect)
 constexpr int kIdleRounds = 8;  // x 4 polls of the host ring before an idle leader goes round its main loop again
 enum RunStatus : int { kRunDone = 0, kRunPreempted = 1 };
 
@@ -75,7 +76,6 @@ struct WgShared {
   uint32_t traceCount;
   uint32_t wgIndex;
   uint32_t round;          // scheduler rounds since launch
-  int32_t express;         // the submission just ingested qualifies for the express path
   int32_t rankBusy;        // leader: other channels of the rank still have work in flight
   int32_t allFresh;        // every collective of the task queue was ingested this round (nothing is parked)
   uint64_t cqNext;         // single-channel ranks: next completion ticket
@@ -85,12 +85,9 @@ struct WgShared {
   int32_t peersLoaded;
   int32_t released;        // the results of this visit are already visible to the system
   int64_t threshold;
-  int64_t slicesSinceLoad;
   CollPlan plan;
   DynCtx dyn;
   WgStats stats;
-  uint64_t peerSend[kMaxDirectRanks];  // direct protocol: the buffers the ranks have published
-  uint64_t peerRecv[kMaxDirectRanks];
   SweepGeom sweep;         // arguments of the direct protocol's sweeps
   uint64_t ticket[2];      // tile numbers handed from thread 0 to the workgroup (two slots, used alternately)
   uint64_t ready[kReadyWords];
@@ -123,6 +120,13 @@ struct WgShared {
 // lanes that run as threads of their own take lane 0's.
 #ifndef DFCCL_WAVE_UNIFORM
 #define DFCCL_WAVE_UNIFORM(x) (x)
+#endif
+
+// Test hook of the host build: a workgroup that never leaves (it ignores the host's requests, quit entries and
+// the idle limit while it keeps running through its own bounded waits), to exercise the host's handling of a
+// kernel that stays resident.  Nothing on the GPU.
+#ifndef DFCCL_TEST_NEVER_LEAVES
+#define DFCCL_TEST_NEVER_LEAVES() false
 #endif
 
 #define DFCCL_AGENT __HIP_MEMORY_SCOPE_AGENT
@@ -234,6 +238,7 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
   // buffers named by the new entries may have been written by the host, a copy engine or another kernel
   // before the submission
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+  const int base = sh.numActive;  // (read by every lane before the ballots below, written by lane 0 after them)
   bool isQuit = false, mine = false;
   if (lane < avail) {
     isQuit = (flags & kSqeFlagQuit) != 0;
@@ -244,8 +249,6 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
   const int take = avail < q ? avail : q;
   const uint64_t mm = __ballot(mine && lane < take);
   const int pos = __builtin_popcountll(mm & ((1ull << lane) - 1ull));
-  const int base = sh.numActive;
-  bool expressLane = false;
   if (mine && lane < take && base + pos < kMaxColls) {
     DFCCL_GLOBAL DynCtx* d = G(&R.dyn[(size_t)ch * R.nColls + coll]);
     d->sendbuff = sendbuff;
@@ -264,12 +267,6 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
         __hip_atomic_store(G(&myPub->send), sendbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
         __hip_atomic_store(G(&myPub->recv), recvbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
         sh.dyn.slice = 1;
-        // alone in the queue and small: wave 0 can run it on the spot (see runExpress)
-        if (base == 0 && __builtin_popcountll(mm) == 1 && sh.plan.kind == kAllReduce && sh.plan.nChannels == 1 &&
-            sh.plan.loopsPerInstance == 1 &&
-            sh.plan.lastChunkElems * sh.plan.elemSize <= kExpressMaxBytes && A.knobs.forceQuitEvery == 0 &&
-            A.knobs.express != 0 && sh.dyn.step == 0)
-          expressLane = true;
       }
     } else {
       // Any other all-reduce of the direct protocol publishes its buffers here as well, straight from the
@@ -288,16 +285,15 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
     }
     sh.taskq[base + pos] = (uint16_t)coll;
   }
-  const bool express = __ballot(expressLane) != 0;
   if (lane == 0) {
-    const int added = __builtin_popcountll(mm);
+    int added = __builtin_popcountll(mm);
+    if (added > kMaxColls - base) added = kMaxColls - base;  // (only the entries that were stored above)
     sh.numActive = base + added;
     const int consumed = take + (q < avail ? 1 : 0);
     sh.frontier += (uint64_t)consumed;
     if (q < avail) sh.finalQuit = 1;
     sh.ingested = consumed;
     sh.allFresh = (base == 0) ? 1 : 0;
-    sh.express = express ? 1 : 0;
     sh.stats.sqesRead += (uint64_t)consumed;
     if (R.nChannels > 1) __hip_atomic_store(G(&R.wgFrontier[ch]), sh.frontier, __ATOMIC_RELAXED, DFCCL_AGENT);
     trace(A, sh, kTrIngested, (uint32_t)consumed);
@@ -495,21 +491,33 @@ __device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, int ch
   DFCCL_WAVE_LDS_SYNC();
 }
 
+// Outcome of a bounded wait.  `ok` comes from a ballot, so every lane of the wave holds the same value in a
+// register: the wave's own code branches on that, never on a copy in LDS (a flag that lane 0 writes and the
+// other lanes of the same wave read back is a data race as far as the compiler can tell, and it has been seen to
+// place the other lanes' read before lane 0's write).  The other waves of the workgroup read sh.waitOk, after a
+// workgroup barrier.
+struct WaitResult {
+  bool ok;
+  uint64_t word;  // the word this lane saw last
+};
+
 // Wave 0: wait until both conditions hold.  Lanes 0..31 watch the counters of
 // w0, lanes 32..63 those of w1; the ballot decides for the whole wave.  The wait
 // is bounded: when the budget is spent the collective is preempted.  (Role of
-// waitPeer, src/collectives_ofccl/device/ofccl_prims_simple.h:90-198.)  Returns the word the lane saw last.
-__device__ __forceinline__ uint64_t waitDescs(const DaemonArgs& A, WgShared& sh, int lane, const WaitDesc& w0,
-                                              const WaitDesc& w1, bool adapt, int64_t cap = 0) {
+// waitPeer, src/collectives_ofccl/device/ofccl_prims_simple.h:90-198.)
+// `threshold` is the visit's spin budget, held in registers by every lane (all lanes update it alike);
+// `slicesSinceLoad` is what the visit has moved so far (only the forced-preemption hook looks at it).
+__device__ __forceinline__ WaitResult waitDescs(const DaemonArgs& A, WgShared& sh, int lane, const WaitDesc& w0,
+                                                const WaitDesc& w1, bool adapt, int64_t& threshold,
+                                                int64_t slicesSinceLoad, int64_t cap = 0) {
   bool ok;
   int64_t spins = 0;
   uint64_t seen = 0;
-  DFCCL_WAVE_LDS_SYNC();  // (what thread 0 wrote before the call is read by every lane below)
   if (lane == 0) trace(A, sh, kTrWaitBegin, (uint32_t)((w0.count + w1.count) & 0xffff));
   const int64_t forceEvery = A.knobs.forceQuitEvery;
-  if (forceEvery > 0 && sh.slicesSinceLoad >= forceEvery) {
+  const bool forced = forceEvery > 0 && slicesSinceLoad >= forceEvery;
+  if (forced) {
     ok = false;
-    if (lane == 0) sh.stats.forcedQuits++;
   } else {
     const WaitDesc& w = (lane < 32) ? w0 : w1;
     const int idx = lane & 31;
@@ -519,33 +527,36 @@ __device__ __forceinline__ uint64_t waitDescs(const DaemonArgs& A, WgShared& sh,
       p = (const DFCCL_GLOBAL uint64_t*)(uintptr_t)(w.ptr + (uint64_t)((int64_t)idx * w.stride));
     const uint64_t need = w.value;
     bool ready = (p == nullptr);
-    const int64_t threshold = (cap > 0 && cap < sh.threshold) ? cap : sh.threshold;
+    const int64_t limit = (cap > 0 && cap < threshold) ? cap : threshold;
     for (;;) {
       if (!ready) {
         seen = __hip_atomic_load(p, __ATOMIC_RELAXED, DFCCL_AGENT);
         ready = waitReached(seen, need, tagged);
       }
       if (__ballot(!ready) == 0) { ok = true; break; }
-      if (++spins >= threshold) { ok = false; break; }
+      if (++spins >= limit) { ok = false; break; }
       __builtin_amdgcn_s_sleep(1);
     }
     if (ok) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  }
+  if (ok && adapt && cap == 0) {
+    const int64_t t = A.knobs.recvSuccessFactor * spins;
+    if (t > threshold) threshold = t;
   }
   if (lane == 0) {
     trace(A, sh, kTrWaitEnd, (uint32_t)((ok ? 1u : 0u) | ((uint32_t)spins << 1)));
     sh.waitOk = ok ? 1 : 0;
     sh.stats.spins += (uint64_t)spins;
-    if (ok && adapt && cap == 0) {
-      const int64_t t = A.knobs.recvSuccessFactor * spins;
-      if (t > sh.threshold) sh.threshold = t;
-    }
+    if (forced) sh.stats.forcedQuits++;
     if (!ok) {
       sh.dyn.wait[0] = w0;
       sh.dyn.wait[1] = w1;
     }
   }
-  DFCCL_WAVE_LDS_SYNC();
-  return seen;
+  WaitResult r;
+  r.ok = ok;
+  r.word = seen;
+  return r;
 }
 
 // ---------------------------------------------------------------- data movement
@@ -616,7 +627,7 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
 // before it writes it, and no other thread touches that pack.
 template <int DT, int OP, int NS>
 __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks], const uint64_t (&dst)[kMaxDirectRanks],
-                                         int n, int nd, int64_t byteOff, size_t nbytes, int tid) {
+                                         int n, int nd, int64_t byteOff, size_t nbytes, int tid, int nthr) {
   constexpr int ES = typeSize(DT);
   uint64_t align = (uint64_t)byteOff;
 #pragma unroll
@@ -627,7 +638,7 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
   if ((align & 15u) == 0) {
     const size_t npacks = nbytes >> 4;
 #pragma clang loop vectorize(disable) interleave(disable) unroll(disable)
-    for (size_t i = tid; i < npacks; i += kWgThreads) {
+    for (size_t i = tid; i < npacks; i += nthr) {
       u32x4 v[NS];
 #pragma unroll
       for (int j = 0; j < NS; j++) v[j] = loadPack<true>((const char*)(j < n ? src[j] : src[0]) + byteOff, i);
@@ -643,7 +654,7 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
   }
   const size_t first = doneBytes / ES, nelem = nbytes / ES;
 #pragma clang loop vectorize(disable) interleave(disable) unroll(disable)
-  for (size_t i = first + tid; i < nelem; i += kWgThreads) {
+  for (size_t i = first + tid; i < nelem; i += nthr) {
     uint32_t acc = loadElem<ES>((const char*)src[0] + byteOff, i);
 #pragma unroll
     for (int j = 1; j < NS; j++)
@@ -668,7 +679,7 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
 // At most maxTiles tiles are processed; `finished` says that no tile is left.
 template <int DT, int OP, int NS>
 __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, int64_t& posInOut, int64_t maxTiles,
-                                           int tid, int64_t& tilesDone, bool& finished) {
+                                           int tid, int nthr, int64_t& tilesDone, bool& finished) {
   const bool dynamic = g.C > 1;
   DFCCL_GLOBAL uint64_t* ctr = (DFCCL_GLOBAL uint64_t*)(uintptr_t)g.ctr;
   int64_t pos = posInOut, done = 0;
@@ -703,7 +714,7 @@ __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, 
     const int64_t real = ((int64_t)l == g.L - 1) ? g.lastReal : g.chunkElems;
     const int64_t off = (int64_t)l * g.loop + ((int64_t)slot * g.tn + g.tme) * real;
     const int64_t nelem = (g.count - off < real) ? g.count - off : real;
-    if (nelem > 0) foldTile<DT, OP, NS>(g.src, g.dst, g.n, g.nd, off * g.es, (size_t)(nelem * g.es), tid);
+    if (nelem > 0) foldTile<DT, OP, NS>(g.src, g.dst, g.n, g.nd, off * g.es, (size_t)(nelem * g.es), tid, nthr);
     done++;
     if (prefetch) {
       if (tid == 0) slots[par] = nxt;
@@ -720,43 +731,37 @@ __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, 
 
 template <int DT, int OP>
 __device__ __forceinline__ void sweepFold(const SweepGeom& g, uint64_t* slots, int64_t& pos, int64_t maxTiles, int tid,
-                                          int64_t& tilesDone, bool& finished) {
-  if (g.n <= 2) sweepFoldN<DT, OP, 2>(g, slots, pos, maxTiles, tid, tilesDone, finished);
-  else if (g.n <= 4) sweepFoldN<DT, OP, 4>(g, slots, pos, maxTiles, tid, tilesDone, finished);
-  else sweepFoldN<DT, OP, 8>(g, slots, pos, maxTiles, tid, tilesDone, finished);
+                                          int nthr, int64_t& tilesDone, bool& finished) {
+  if (g.n <= 2) sweepFoldN<DT, OP, 2>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
+  else if (g.n <= 4) sweepFoldN<DT, OP, 4>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
+  else sweepFoldN<DT, OP, 8>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
 }
 
 template <int DT>
 __device__ __forceinline__ void sweepFoldOp(int op, const SweepGeom& g, uint64_t* slots, int64_t& pos, int64_t maxTiles,
-                                            int tid, int64_t& tilesDone, bool& finished) {
+                                            int tid, int nthr, int64_t& tilesDone, bool& finished) {
   switch (op) {
-    case kSum: sweepFold<DT, kSum>(g, slots, pos, maxTiles, tid, tilesDone, finished); break;
-    case kProd: sweepFold<DT, kProd>(g, slots, pos, maxTiles, tid, tilesDone, finished); break;
-    case kMax: sweepFold<DT, kMax>(g, slots, pos, maxTiles, tid, tilesDone, finished); break;
-    default: sweepFold<DT, kMin>(g, slots, pos, maxTiles, tid, tilesDone, finished); break;
+    case kSum: sweepFold<DT, kSum>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
+    case kProd: sweepFold<DT, kProd>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
+    case kMax: sweepFold<DT, kMax>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
+    default: sweepFold<DT, kMin>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
   }
 }
 
-// The geometry and the buffer tables are handed over in LDS and copied to registers here.
-__device__ __forceinline__ void sweepFoldAny(const SweepGeom* gp, uint64_t* slots, int64_t& pos, int64_t maxTiles,
-                                             int tid, int64_t& tilesDone, bool& finished) {
-  SweepGeom g = *gp;
-#pragma unroll
-  for (int t = 0; t < kMaxDirectRanks; t++) {
-    g.src[t] = uniform64(g.src[t]);
-    g.dst[t] = uniform64(g.dst[t]);
-  }
+// `tid` of `nthr` threads take part (the whole workgroup, or wave 0 alone); the geometry is the same in all of them.
+__device__ __forceinline__ void sweepFoldAny(const SweepGeom& g, uint64_t* slots, int64_t& pos, int64_t maxTiles,
+                                             int tid, int nthr, int64_t& tilesDone, bool& finished) {
   const int op = g.op;
   if (g.n <= 1) {  // plain copy, whatever the type
-    sweepFoldN<kI8, kSum, 1>(g, slots, pos, maxTiles, tid, tilesDone, finished);
+    sweepFoldN<kI8, kSum, 1>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
     return;
   }
   switch (g.dtype) {
-    case kF32: sweepFoldOp<kF32>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
-    case kBF16: sweepFoldOp<kBF16>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
-    case kF16: sweepFoldOp<kF16>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
-    case kI32: sweepFoldOp<kI32>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
-    default: sweepFoldOp<kI8>(op, g, slots, pos, maxTiles, tid, tilesDone, finished); break;
+    case kF32: sweepFoldOp<kF32>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
+    case kBF16: sweepFoldOp<kBF16>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
+    case kF16: sweepFoldOp<kF16>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
+    case kI32: sweepFoldOp<kI32>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
+    default: sweepFoldOp<kI8>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
   }
 }
 
@@ -784,6 +789,8 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
   int64_t grid = sh.dyn.gridOffset;
   int step0 = sh.dyn.step, slice0 = sh.dyn.slice;
   uint64_t sendStep = sh.dyn.sendStep, recvStep = sh.dyn.recvStep;
+  int64_t threshold = sh.threshold;  // the visit's spin budget (every thread keeps the same copy)
+  int64_t slicesSinceLoad = 0;       // slices this visit has moved
 
   for (; grid < count; grid += loop, step0 = 0) {
     const int64_t real = realChunkElems(kind, n, C, P.chunkElems, P.alignElems, count, grid);
@@ -799,9 +806,11 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
           const WaitDesc w0 = d.recv ? waitFor(&P.recvFlags[ch].tail, recvStep + 1, 0, 1) : noWait();
           const uint64_t needHead = (sendStep + 1 > (uint64_t)P.fifoSlots) ? sendStep + 1 - (uint64_t)P.fifoSlots : 0;
           const WaitDesc w1 = d.send ? waitFor(&P.sendFlags[ch].head, needHead, 0, 1) : noWait();
-          if (wave == 0) waitDescs(A, sh, lane, w0, w1, d.recv != 0);
+          bool ok = true;
+          if (wave == 0) ok = waitDescs(A, sh, lane, w0, w1, d.recv != 0, threshold, slicesSinceLoad).ok;
           __syncthreads();
-          if (!sh.waitOk) {
+          if (wave != 0) ok = sh.waitOk != 0;
+          if (!ok) {
             if (tid == 0) {
               sh.dyn.gridOffset = grid;
               sh.dyn.step = s;
@@ -831,9 +840,9 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
             if (d.recv) __hip_atomic_store(G(&P.recvFlags[ch].head), recvStep + 1, __ATOMIC_RELAXED, DFCCL_AGENT);
             trace(A, sh, kTrPosted, (uint32_t)s);
             sh.progressed = 1;
-            sh.slicesSinceLoad++;
             sh.stats.slicesMoved++;
           }
+          slicesSinceLoad++;
           sendStep += d.send ? 1 : 0;
           recvStep += d.recv ? 1 : 0;
         } else if (tid == 0) {
@@ -851,6 +860,56 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
 }
 
 // ----------------------------------------------------------------- direct protocol
+
+// The value lane `srcLane` of the wave holds (srcLane is the same in every lane): a register read, no LDS.
+__device__ __forceinline__ uint64_t readLane64(uint64_t v, int srcLane) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, srcLane);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), srcLane);
+  return (uint64_t)lo | ((uint64_t)hi << 32);
+}
+
+// Wave 0, after the wait for the peers' publications: lanes 0..n-1 hold the peers' send words, lanes
+// 32..32+n-1 their receive words.  Every lane builds the whole geometry of the sweep in registers.
+__device__ __forceinline__ void layOutSweep(SweepGeom& g, const CollPlan& P, int ch, uint64_t inst, uint64_t word) {
+  const int kind = P.kind, root = P.root, n = P.nRanks, me = P.rank, C = P.nChannels, es = P.elemSize;
+  const int64_t L = P.loopsPerInstance;
+  const bool owned = (kind == kAllReduce || kind == kReduce || kind == kBroadcast);
+  const bool folds = (kind == kAllReduce || kind == kReduce || kind == kReduceScatter);
+  const bool toAll = (kind == kAllReduce || kind == kBroadcast || kind == kAllGather);
+  const int first = ((kind == kReduce) ? root : me) + 1;  // rank the fold starts with (before wrapping)
+  const uint64_t srcOff = (kind == kReduceScatter) ? (uint64_t)me * (uint64_t)P.count * (uint64_t)es : 0;
+  const uint64_t dstOff = (kind == kAllGather) ? (uint64_t)me * (uint64_t)P.count * (uint64_t)es : 0;
+  g.n = folds ? n : 1;
+  g.nd = toAll ? n : 1;
+#pragma unroll
+  for (int t = 0; t < kMaxDirectRanks; t++) {
+    int sr = folds ? first + t : (kind == kBroadcast ? root : me);
+    if (sr >= n) sr -= n;
+    if (sr >= n) sr = 0;  // (t >= n: the entry is not used)
+    int dr = toAll ? t : (kind == kReduce ? root : me);
+    if (dr >= n) dr = 0;
+    const uint64_t sp = readLane64(word, sr) & kPtrMask, dp = readLane64(word, 32 + dr) & kPtrMask;
+    g.src[t] = (t < g.n) ? sp + srcOff : 0;
+    g.dst[t] = (t < g.nd) ? dp + dstOff : 0;
+  }
+  g.tn = owned ? n : 1;
+  g.tme = owned ? me : 0;
+  g.count = P.count;
+  g.loop = (int64_t)C * g.tn * P.chunkElems;
+  g.chunkElems = P.chunkElems;
+  g.lastReal = P.lastChunkElems;
+  g.L = L;
+  g.T = L * C;
+  g.instBase = inst * (uint64_t)(L * C);
+  g.ctr = (uint64_t)(uintptr_t)P.tileCtr;
+  g.C = C;
+  g.ch = ch;
+  g.es = es;
+  g.me = me;
+  g.dtype = P.dtype;
+  g.op = P.op;
+  g.pad0 = g.pad1 = 0;
+}
 
 // Collectives in which the virtual ranks, whose buffers share one HBM, read each
 // other's send buffers and write each other's receive buffers in place.
@@ -877,26 +936,42 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
 // dyn.step is the phase (0 = sweep, 2 = only the final wait is left),
 // dyn.gridOffset the sweep's position (see sweepFoldN), dyn.slice whether the
 // instance is published.
+//
+// Small collectives (the low-latency path): when the whole share of this rank is one tile of at most
+// kSoloMaxBytes, wave 0 runs the instance alone (`solo`): waits, sweep, release and the final wait follow each
+// other inside one wave, with every decision in registers and not one workgroup barrier in between, while the
+// other waves go straight to the barrier that ends the visit.  The steps, the memory ordering and the saved
+// state are the same as for the whole workgroup; only who takes part differs.
 __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
   const CollPlan& P = sh.plan;
   const int lane = tid & 63, wave = tid >> 6;
-  const int n = P.nRanks, C = P.nChannels, es = P.elemSize, me = P.rank;
-  const int64_t count = P.count;
+  const int n = P.nRanks, C = P.nChannels, me = P.rank;
   const int64_t L = P.loopsPerInstance;
+  const int64_t forceEvery = A.knobs.forceQuitEvery;
+  const bool solo = C == 1 && L == 1 && forceEvery == 0 && P.lastChunkElems * P.elemSize <= kSoloMaxBytes;
+  // (the plan does not change during a visit, so every wave decides alike; what the other waves return is not
+  // looked at: thread 0 reports the outcome)
+  if (solo && wave != 0) return kRunDone;
+  const int nthr = solo ? 64 : kWgThreads;   // threads that take part from here on
+  const int mtid = solo ? lane : tid;
+
   const uint64_t inst = sh.dyn.instance;
   const uint64_t base = inst * (uint64_t)L;
   const uint64_t sendbuff = sh.dyn.sendbuff, recvbuff = sh.dyn.recvbuff;
   const int published = sh.dyn.slice;
-  const int peersLoaded = sh.peersLoaded;
+  const int peersLoaded = solo ? 0 : sh.peersLoaded;  // (a wave on its own keeps the sweep's geometry in registers)
   const int pubStride = C * (int)sizeof(PeerPub), ctrStride = C * 8;
-  const int64_t forceEvery = A.knobs.forceQuitEvery;
   PeerPub* myPub = &P.pubs[(size_t)me * C + ch];
   const int64_t l0 = sh.dyn.gridOffset;
   const int phase = sh.dyn.step;
+  int64_t threshold = sh.threshold;  // the visit's spin budget (every thread keeps the same copy)
+  int64_t slicesSinceLoad = 0;       // tiles this visit has moved
   // With other collectives queued a wait is only a look: switching is cheap here (contexts are small and
   // nothing is held while parked), and the workgroup is better off moving the next collective's data.
   const int64_t cap = (sh.numActive > 1 && forceEvery == 0) ? kSoftWaitSpins : 0;
-  __syncthreads();  // every thread has taken its copy of the position before thread 0 changes it
+  // every thread has taken its copy of the position before thread 0 changes it
+  if (solo) DFCCL_WAVE_LDS_SYNC();
+  else __syncthreads();
 
   if (!published && tid < 2) {
     // the words carry their own instance tag: no ordering between them is needed, and the buffers' contents
@@ -908,57 +983,34 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
   }
 
   if (phase == 0) {
+    SweepGeom g;
     if (!peersLoaded) {
-      // lanes 0..n-1 watch the peers' send words, lanes 32..32+n-1 their receive words
-      const WaitDesc w0 = waitFor(&P.pubs[ch].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
-      const WaitDesc w1 = waitFor(&P.pubs[ch].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
+      bool ok = true;
       if (wave == 0) {
-        const uint64_t word = waitDescs(A, sh, lane, w0, w1, true, cap);
-        if (sh.waitOk && (lane & 31) < n) {
-          if (lane < 32) sh.peerSend[lane] = word & kPtrMask;
-          else sh.peerRecv[lane & 31] = word & kPtrMask;
-        }
-        DFCCL_WAVE_LDS_SYNC();
-        if (sh.waitOk && lane == 0) {
-          SweepGeom& g = sh.sweep;
-          const int kind = P.kind, root = P.root;
-          const bool owned = (kind == kAllReduce || kind == kReduce || kind == kBroadcast);
-          const bool folds = (kind == kAllReduce || kind == kReduce || kind == kReduceScatter);
-          const bool toAll = (kind == kAllReduce || kind == kBroadcast || kind == kAllGather);
-          const int first = (kind == kReduce) ? root + 1 : me + 1;  // rank the fold starts with
-          const uint64_t srcOff = (kind == kReduceScatter) ? (uint64_t)me * (uint64_t)count * (uint64_t)es : 0;
-          const uint64_t dstOff = (kind == kAllGather) ? (uint64_t)me * (uint64_t)count * (uint64_t)es : 0;
-          g.n = folds ? n : 1;
-          g.nd = toAll ? n : 1;
-          for (int t = 0; t < kMaxDirectRanks; t++) {
-            uint64_t sp = 0, dp = 0;
-            if (t < g.n) sp = sh.peerSend[folds ? (first + t) % n : (kind == kBroadcast ? root : me)] + srcOff;
-            if (t < g.nd) dp = sh.peerRecv[toAll ? t : (kind == kReduce ? root : me)] + dstOff;
-            g.src[t] = sp;
-            g.dst[t] = dp;
+        // lanes 0..n-1 watch the peers' send words, lanes 32..32+n-1 their receive words
+        const WaitDesc w0 = waitFor(&P.pubs[ch].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
+        const WaitDesc w1 = waitFor(&P.pubs[ch].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
+        const WaitResult r = waitDescs(A, sh, lane, w0, w1, true, threshold, slicesSinceLoad, cap);
+        ok = r.ok;
+        if (ok) {
+          layOutSweep(g, P, ch, inst, r.word);
+          if (!solo && lane == 0) {
+            sh.sweep = g;  // for the other waves, and for a later visit that finds the context still resident
+            sh.peersLoaded = 1;
           }
-          g.tn = owned ? n : 1;
-          g.tme = owned ? me : 0;
-          g.count = count;
-          g.loop = (int64_t)C * g.tn * P.chunkElems;
-          g.chunkElems = P.chunkElems;
-          g.lastReal = P.lastChunkElems;
-          g.L = L;
-          g.T = L * C;
-          g.instBase = inst * (uint64_t)(L * C);
-          g.ctr = (uint64_t)(uintptr_t)P.tileCtr;
-          g.C = C;
-          g.ch = ch;
-          g.es = es;
-          g.me = me;
-          g.dtype = P.dtype;
-          g.op = P.op;
-          g.pad0 = g.pad1 = 0;
-          sh.peersLoaded = 1;
         }
       }
-      __syncthreads();
-      if (!sh.waitOk) return kRunPreempted;  // position unchanged
+      if (!solo) {
+        __syncthreads();
+        if (wave != 0) ok = sh.waitOk != 0;
+      }
+      if (!ok) return kRunPreempted;  // position unchanged
+    }
+    if (!solo) g = sh.sweep;
+#pragma unroll
+    for (int t = 0; t < kMaxDirectRanks; t++) {
+      g.src[t] = uniform64(g.src[t]);
+      g.dst[t] = uniform64(g.dst[t]);
     }
 
     if (tid == 0) trace(A, sh, kTrMoveBegin, 0);
@@ -967,9 +1019,8 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
     if (forceEvery > 0) {
       // test hook: one tile at a time, with a preemption point before each
       while (!finished) {
-        __syncthreads();
-        if (sh.slicesSinceLoad >= forceEvery) {
-          __syncthreads();
+        __syncthreads();  // (the previous tile's ticket has been read by everybody before it is handed out again)
+        if (slicesSinceLoad >= forceEvery) {
           if (tid == 0) {
             sh.stats.forcedQuits++;
             sh.dyn.gridOffset = pos;
@@ -979,27 +1030,28 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
           }
           return kRunPreempted;
         }
-        __syncthreads();
-        sweepFoldAny(&sh.sweep, sh.ticket, pos, 1, tid, tilesDone, finished);
+        sweepFoldAny(g, sh.ticket, pos, 1, mtid, nthr, tilesDone, finished);
+        slicesSinceLoad += tilesDone;
         if (tid == 0 && tilesDone > 0) {
           sh.progressed = 1;
-          sh.slicesSinceLoad += tilesDone;
           sh.stats.slicesMoved += (uint64_t)tilesDone;
         }
       }
     } else {
-      sweepFoldAny(&sh.sweep, sh.ticket, pos, INT64_MAX, tid, tilesDone, finished);
+      sweepFoldAny(g, sh.ticket, pos, INT64_MAX, mtid, nthr, tilesDone, finished);
       if (tid == 0) {
         sh.progressed = 1;
-        sh.slicesSinceLoad += tilesDone;
         sh.stats.slicesMoved += (uint64_t)tilesDone;
       }
     }
-    __syncthreads();
+    // Released to the system here, while the peers are still busy, so that the completion need not wait for it.
+    // Whole workgroup: the barrier orders every thread's stores before thread 0's fence.  Wave 0 alone: every
+    // lane's stores are covered by the fence the wave executes together.
+    if (solo) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+    else __syncthreads();
     if (tid == 0) {
       trace(A, sh, kTrMoveEnd, 0);
-      // released to the system here, while the peers are still busy, so that the completion need not wait for it
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+      if (!solo) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
       sh.released = 1;
       __hip_atomic_store(G(&P.p1[(size_t)me * C + ch]), base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
       trace(A, sh, kTrPosted, 1);
@@ -1010,9 +1062,13 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
   if (phase != 0 && tid == 0) sh.released = 1;  // resumed here: the sweep's release was done before it was parked
   {
     const WaitDesc w0 = waitFor(&P.p1[ch], base + (uint64_t)L, ctrStride, n);
-    if (wave == 0) waitDescs(A, sh, lane, w0, noWait(), true, cap);
-    __syncthreads();
-    if (!sh.waitOk) {
+    bool ok = true;
+    if (wave == 0) ok = waitDescs(A, sh, lane, w0, noWait(), true, threshold, slicesSinceLoad, cap).ok;
+    if (!solo) {
+      __syncthreads();
+      if (wave != 0) ok = sh.waitOk != 0;
+    }
+    if (!ok) {
       if (tid == 0) {
         sh.dyn.gridOffset = 0;
         sh.dyn.step = 2;
@@ -1069,123 +1125,6 @@ __device__ __forceinline__ void completeColl(const DaemonArgs& A, const RankDev&
   storeStruct(&R.dyn[(size_t)ch * R.nColls + coll], sh.dyn);
 }
 
-template <int DT>
-__device__ __forceinline__ u32x4 foldPacksOp(int op, const u32x4 (&v)[kMaxDirectRanks], int n) {
-  u32x4 acc = v[0];
-#pragma unroll
-  for (int t = 1; t < kMaxDirectRanks; t++) {
-    if (t < n) {
-      switch (op) {
-        case kSum: acc = packOp<DT, kSum>(acc, v[t]); break;
-        case kProd: acc = packOp<DT, kProd>(acc, v[t]); break;
-        case kMax: acc = packOp<DT, kMax>(acc, v[t]); break;
-        default: acc = packOp<DT, kMin>(acc, v[t]); break;
-      }
-    }
-  }
-  return acc;
-}
-
-// The express path for small all-reduces, run by wave 0 alone inside the ingest phase: when the submission
-// that just arrived is the only work of the workgroup, is the next instance of the resident collective (so
-// its buffers have been published at ingest already), uses the direct protocol on one channel in one loop
-// and this rank's chunk is at most kExpressMaxBytes, the wave does the whole instance (wait for the peers'
-// buffers, fold, store everywhere, release, wait for the peers, post the completion) without a workgroup
-// barrier and without going through the scheduler.  A wait that runs out of budget, or buffers that are not
-// 16-byte aligned, hand the collective to the scheduler in the state it has reached.  Returns true if the
-// instance is complete.
-__device__ __forceinline__ bool runExpress(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane) {
-  const CollPlan& P = sh.plan;
-  const uint32_t coll = sh.taskq[0];
-  const int n = P.nRanks, es = P.elemSize, me = P.rank;
-  const uint64_t inst = sh.dyn.instance;
-  const int pubStride = (int)sizeof(PeerPub);  // one channel
-  if (lane == 0) {
-    sh.threshold = A.knobs.baseCtxSwitchThreshold * A.knobs.numTryTaskqHead;
-    if (sh.threshold < 1) sh.threshold = 1;
-    sh.waitOk = 1;
-    sh.released = 0;
-    sh.slicesSinceLoad = 0;
-    trace(A, sh, kTrVisitBegin, coll);
-  }
-  DFCCL_WAVE_LDS_SYNC();
-  // lanes 0..n-1 get the peers' send buffers, lanes 32..32+n-1 their receive buffers
-  const WaitDesc w0 = waitFor(&P.pubs[0].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
-  const WaitDesc w1 = waitFor(&P.pubs[0].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
-  const uint64_t word = waitDescs(A, sh, lane, w0, w1, false) & kPtrMask;
-  if (!sh.waitOk) return false;  // nothing done yet: the scheduler starts from the published state
-  const int64_t real = P.lastChunkElems;
-  const int64_t off = (int64_t)me * real;
-  int64_t nelem = (P.count - off < real) ? P.count - off : real;
-  if (nelem < 0) nelem = 0;
-  const int64_t byteOff = off * es;
-  const size_t nbytes = (size_t)(nelem * es);
-  // every pointer and the length must allow 128-bit accesses
-  uint64_t misaligned = ((lane & 31) < n) ? (word & 15u) : 0;
-  misaligned |= (uint64_t)(nbytes & 15u);
-  if (__ballot(misaligned != 0) != 0) return false;
-  if (lane == 0) trace(A, sh, kTrMoveBegin, 0);
-  uint64_t src[kMaxDirectRanks], dst[kMaxDirectRanks];
-#pragma unroll
-  for (int t = 0; t < kMaxDirectRanks; t++) {
-    int r = me + 1 + t;  // fold order in[me + 1], in[me + 2], ..., in[me]; surplus entries repeat the first
-    if (t >= n) r = me + 1;
-    if (r >= n) r -= n;
-    src[t] = uniform64(__shfl(word, r));
-    dst[t] = uniform64(__shfl(word, 32 + (t < n ? t : 0)));
-  }
-  const size_t npacks = nbytes >> 4;
-  for (size_t i = lane; i < npacks; i += 64) {
-    u32x4 v[kMaxDirectRanks];
-#pragma unroll
-    for (int t = 0; t < kMaxDirectRanks; t++) v[t] = loadPack<true>((const char*)src[t] + byteOff, i);
-    u32x4 acc;
-    switch (P.dtype) {
-      case kF32: acc = foldPacksOp<kF32>(P.op, v, n); break;
-      case kBF16: acc = foldPacksOp<kBF16>(P.op, v, n); break;
-      case kF16: acc = foldPacksOp<kF16>(P.op, v, n); break;
-      case kI32: acc = foldPacksOp<kI32>(P.op, v, n); break;
-      default: acc = foldPacksOp<kI8>(P.op, v, n); break;
-    }
-#pragma unroll
-    for (int t = 0; t < kMaxDirectRanks; t++)
-      if (t < n) storePack<false>((char*)dst[t] + byteOff, i, acc);
-  }
-  // all lanes' stores are covered by the wave's release
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-  if (lane == 0) {
-    trace(A, sh, kTrMoveEnd, 0);
-    sh.released = 1;
-    __hip_atomic_store(G(&P.p1[me]), inst + 1, __ATOMIC_RELAXED, DFCCL_AGENT);  // one loop per instance
-    trace(A, sh, kTrPosted, 1);
-    sh.progressedRound = 1;
-    sh.stats.slicesMoved++;
-  }
-  DFCCL_WAVE_LDS_SYNC();
-  const WaitDesc wp = waitFor(&P.p1[0], inst + 1, 8, n);
-  waitDescs(A, sh, lane, wp, noWait(), false);
-  if (!sh.waitOk) {
-    // the scheduler takes over at the final wait (waitDescs has stored what the collective is parked on)
-    if (lane == 0) {
-      sh.dyn.gridOffset = 0;
-      sh.dyn.step = 2;
-      sh.stats.ctxSaves++;
-      storeStruct(&R.dyn[(size_t)ch * R.nColls + coll], sh.dyn);
-    }
-    DFCCL_WAVE_LDS_SYNC();
-    return false;
-  }
-  if (lane == 0) {
-    sh.dyn.instance = inst + 1;
-    sh.dyn.slice = 0;
-    completeColl(A, R, sh, ch, coll);
-    sh.numActive = 0;
-    trace(A, sh, kTrVisitEnd, 0);
-  }
-  DFCCL_WAVE_LDS_SYNC();
-  return true;
-}
-
 // Visit one collective of the task queue: make its context resident, run it,
 // then post the completion or save the context.
 __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int tid, int qi) {
@@ -1209,7 +1148,6 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
     sh.waitOk = 1;
     sh.progressed = 0;
     sh.released = 0;
-    sh.slicesSinceLoad = 0;
     sh.dyn.wait[0] = noWait();
     sh.dyn.wait[1] = noWait();
     trace(A, sh, kTrVisitBegin, coll);
@@ -1290,15 +1228,16 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     if (wave == 0) {
       if (ch == 0) pollHost(A, R, sh, lane);
       else ingestMirror(A, R, sh, ch, lane);
-      if (sh.ingested > 0 && sh.express) runExpress(A, R, sh, ch, lane);
       if (sh.numActive > 0) scanReady(R, sh, ch, lane);
       else if (lane == 0) sh.numReady = 0;
       DFCCL_WAVE_LDS_SYNC();
       if (lane == 0) {
-        // the host's requests and the lifetime limit are looked at every 8th round: nobody waits on them
+        // the host's requests and the lifetime limit are looked at every 8th round, and only every 64th while
+        // submissions keep arriving: nobody waits on them, and a new submission does not wait for them either
         uint32_t abortFlag = 0, quitFlag = 0;
         bool expired = false;
-        if ((sh.round++ & 7u) == 0) {
+        const uint32_t round = sh.round++;
+        if ((round & 7u) == 0 && (sh.ingested == 0 || (round & 63u) == 0)) {
           abortFlag = __hip_atomic_load(G(&A.devFlags[1]), __ATOMIC_RELAXED, DFCCL_AGENT);
           quitFlag = __hip_atomic_load(G(&A.devFlags[0]), __ATOMIC_RELAXED, DFCCL_AGENT);
           const uint32_t statsReq = __hip_atomic_load(G(&A.devFlags[2]), __ATOMIC_RELAXED, DFCCL_AGENT);
@@ -1315,7 +1254,15 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
         if (abortFlag) sh.exitKind = kExitAbort;
         else if (sh.finalQuit) sh.exitKind = kExitFinal;
         else if (quitFlag || expired) sh.exitKind = kExitVoluntary;
-        else if (sh.idle >= K.tolerantUnprogressedCnt) sh.exitKind = kExitVoluntary;
+        else if (sh.idle >= K.tolerantUnprogressedCnt) {
+          // Idle for long: leave, and take the whole daemon along (every workgroup saves its state and leaves at
+          // its next look at this flag).  The kernel can only be launched again once all of it has ended, and a
+          // submission for a rank whose workgroups have left is not seen by anybody until then: a daemon that
+          // stays half resident because other ranks are busy would starve that rank.
+          sh.exitKind = kExitVoluntary;
+          __hip_atomic_store(G(&A.devFlags[0]), 1u, __ATOMIC_RELAXED, DFCCL_AGENT);
+        }
+        if (DFCCL_TEST_NEVER_LEAVES()) sh.exitKind = kExitNone;
         sh.progressedRound = 0;
       }
       DFCCL_WAVE_LDS_SYNC();

@@ -202,7 +202,6 @@ struct Knobs {
   int64_t tolerantUnprogressedCnt;  // TOLERANT_UNPROGRESSED_CNT, default 500000
   int64_t forceQuitEvery;           // DFCCL_FORCE_QUIT_EVERY: preempt after this many slices (0 = off)
   int64_t maxLifetimeTicks;         // DFCCL_DAEMON_MAX_MS in 100 MHz ticks (0 = unlimited)
-  int64_t express;                  // DFCCL_EXPRESS: 1 switches the express path for small all-reduces on
   int64_t idlePollRounds;           // DFCCL_IDLE_POLL_ROUNDS: 0 switches the pipelined polling of idle leaders off
 };
 

@@ -140,6 +140,7 @@ struct ofcclRankCtx {
   // submission side
   std::mutex sqMu;
   uint64_t sqTail = 0;
+  uint64_t sqCapacity = dfccl::kSqCapacity;  // entries that may be outstanding (DFCCL_SQ_CAPACITY lowers it, for tests)
   // completion side
   uint64_t cqRead = 0;
   CallbackFunc callbacks[dfccl::kMaxColls];
@@ -148,6 +149,7 @@ struct ofcclRankCtx {
   uint64_t submitNs[dfccl::kMaxColls];    // steady-clock time the last instance was queued
   uint64_t completeNs[dfccl::kMaxColls];  // steady-clock time its completion entry was seen by the poller
   std::atomic<uint64_t> submitted{0}, completed{0};
+  std::atomic<uint64_t> sqFullSpins{0};  // times a Run found the submission ring full and had to wait
   std::thread poller;
   std::atomic<bool> stopPoller{false};
   std::atomic<bool> pollerAsleep{false};
@@ -170,7 +172,7 @@ struct Daemon {
   bool running = false;
   bool shutdown = false;
   bool launchRequested = false;
-  bool failed = false;
+  std::atomic<bool> failed{false};  // launch failed or the kernel had to be aborted: never launched again
   uint32_t epoch = 0;
   uint64_t launches = 0;
   long capacity = 0;
@@ -221,9 +223,6 @@ struct Daemon {
     knobs.tolerantUnprogressedCnt = envInt("TOLERANT_UNPROGRESSED_CNT", 500000);
     knobs.forceQuitEvery = envInt("DFCCL_FORCE_QUIT_EVERY", 0);
     knobs.maxLifetimeTicks = envInt("DFCCL_DAEMON_MAX_MS", 0) * 100000;  // wall_clock64 runs at 100 MHz
-    // Off unless asked for: its stress test (spin limit 1, every bounded wait gives up) faulted the GPU; the cause
-    // is fixed (see DFCCL_WAVE_LDS_SYNC in daemon.hip) but the test has not been run on a GPU again yet.
-    knobs.express = envInt("DFCCL_EXPRESS", 0);
     knobs.idlePollRounds = envInt("DFCCL_IDLE_POLL_ROUNDS", 8);
     if (knobs.numTryTaskqHead < 1) knobs.numTryTaskqHead = 1;
     if (knobs.tolerantUnprogressedCnt < 1) knobs.tolerantUnprogressedCnt = 1;
@@ -304,9 +303,11 @@ struct Daemon {
       fprintf(stderr, "dfccl: daemon did not leave on request, aborting it\n");
       failed = true;  // the aborted kernel's state is abandoned: no relaunch
       __atomic_store_n(ctrl, kCtrlAbort, __ATOMIC_RELEASE);
-      cv.wait_for(lk, std::chrono::seconds(20), [&] { return !running; });
+      cv.wait_for(lk, std::chrono::milliseconds(abortWaitMs()), [&] { return !running; });
     }
   }
+  // how long an aborted kernel is given to leave (DFCCL_ABORT_WAIT_MS is for tests)
+  static int64_t abortWaitMs() { return std::max<int64_t>(1, envInt("DFCCL_ABORT_WAIT_MS", 10000)); }
 };
 
 // What the host knows about every attached rank, printed before a daemon is aborted (caller holds d->mu).
@@ -339,6 +340,19 @@ static void dumpDaemonState(const Daemon* d) {
   }
 }
 
+// The kernel is still resident although it was told to abort (a workgroup that cannot reach the point where it
+// looks at the flag).  Nothing of the daemon can be freed while it runs, the observer thread is inside
+// hipEventSynchronize and every call that waits for the device would block for good: say what is known and end
+// the process.  Caller holds d->mu.
+[[noreturn]] static void giveUpOnResidentDaemon(const Daemon* d, const char* where) {
+  fprintf(stderr, "dfccl: the daemon kernel on device %d is still resident after an abort request (%s); "
+          "ending the process\n", d->device, where);
+  dumpDaemonState(d);
+  fflush(stderr);
+  fflush(stdout);
+  _exit(70);
+}
+
 static std::mutex gDaemonMu;
 static std::map<int, Daemon*> gDaemons;
 static bool gAtexitRegistered = false;
@@ -351,7 +365,8 @@ static void abortAllDaemonsAtExit() {
     if (d->running) {
       d->failed = true;
       __atomic_store_n(d->ctrl, kCtrlAbort, __ATOMIC_RELEASE);
-      d->cv.wait_for(lk, std::chrono::seconds(5), [&] { return !d->running; });
+      d->cv.wait_for(lk, std::chrono::milliseconds(Daemon::abortWaitMs()), [&] { return !d->running; });
+      if (d->running) giveUpOnResidentDaemon(d, "process exit");
     }
   }
 }
@@ -401,7 +416,8 @@ static void destroyDaemon(Daemon* d) {
       if (!d->cv.wait_for(lk, std::chrono::seconds(10), [&] { return !d->running; })) {
         d->failed = true;
         __atomic_store_n(d->ctrl, kCtrlAbort, __ATOMIC_RELEASE);
-        d->cv.wait_for(lk, std::chrono::seconds(10), [&] { return !d->running; });
+        d->cv.wait_for(lk, std::chrono::milliseconds(Daemon::abortWaitMs()), [&] { return !d->running; });
+        if (d->running) giveUpOnResidentDaemon(d, "freeing the daemon");
       }
     }
     d->shutdown = true;
@@ -617,12 +633,15 @@ static void pollerLoop(ofcclRankCtx* c) {
 // --------------------------------------------------------------------- submission
 
 // Writes one entry to the host-coherent ring (sqWrite, src/enqueue_ofccl.cc:616-656).
-// Returns -1 if the ring is full.
-static int sqWrite(ofcclRankCtx* c, uint64_t sendbuff, uint64_t recvbuff, uint32_t coll, uint32_t flags) {
+// Returns -1 if the ring is full.  `stampNs`, if given, receives the steady-clock time just before the entry
+// becomes visible to the device (so a completion can never be stamped earlier than its submission).
+static int sqWrite(ofcclRankCtx* c, uint64_t sendbuff, uint64_t recvbuff, uint32_t coll, uint32_t flags,
+                   uint64_t* stampNs = nullptr) {
   std::lock_guard<std::mutex> lk(c->sqMu);
   const uint64_t head = __atomic_load_n(c->dev.sqHead, __ATOMIC_ACQUIRE);
-  if (c->sqTail - head >= (uint64_t)kSqCapacity) return -1;
+  if (c->sqTail - head >= c->sqCapacity) return -1;
   const uint64_t t = c->sqTail;
+  if (stampNs) *stampNs = nowNs();
   uint64_t* w = c->dev.sq + (t & (kSqRing - 1)) * kSqeWords;
   const uint64_t tag = sqeTag(t);
   __atomic_store_n(&w[0], (sendbuff & kPtrMask) | tag, __ATOMIC_RELEASE);
@@ -640,23 +659,29 @@ static ncclResult_t runColl(const void* sendbuff, void* recvbuff, int collId, Ca
   if (collId < 0 || collId >= kMaxColls || c->collIndex[collId] < 0) return ncclInvalidArgument;
   if (((uint64_t)(uintptr_t)sendbuff & ~kPtrMask) || ((uint64_t)(uintptr_t)recvbuff & ~kPtrMask))
     return ncclInvalidArgument;
-  // one instance per collId in flight
+  Daemon* d = c->daemon;
+  // one instance per collId in flight: a second Run waits for the first (for ever only if the daemon is lost)
   int expected = 0;
   while (!c->inflight[collId].compare_exchange_weak(expected, 1, std::memory_order_acq_rel)) {
     expected = 0;
+    if (d->failed.load(std::memory_order_acquire)) return ncclSystemError;
     sched_yield();
   }
   c->callbacks[collId] = cb;
   c->cbArgs[collId] = cbArgs;
   c->submitted.fetch_add(1);
-  while (sqWrite(c, (uint64_t)(uintptr_t)sendbuff, (uint64_t)(uintptr_t)recvbuff, (uint32_t)c->collIndex[collId], 0) ==
-         -1) {
+  // a full ring back-pressures the caller (CpuSqFull, src/enqueue_ofccl.h:51-54; the spin of
+  // src/collectives_ofccl/ofccl_all_reduce.cc:29-33)
+  while (sqWrite(c, (uint64_t)(uintptr_t)sendbuff, (uint64_t)(uintptr_t)recvbuff, (uint32_t)c->collIndex[collId], 0,
+                 &c->submitNs[collId]) == -1) {
+    if (d->failed.load(std::memory_order_acquire)) {
+      c->submitted.fetch_sub(1);
+      c->inflight[collId].store(0, std::memory_order_release);
+      return ncclSystemError;
+    }
+    c->sqFullSpins.fetch_add(1, std::memory_order_relaxed);
     sched_yield();
   }
-  // written before the completion can be consumed only in practice (the device round trip takes microseconds);
-  // readers take it after the callback
-  c->submitNs[collId] = nowNs();
-  Daemon* d = c->daemon;
   {
     // wake the observer if the kernel is not resident (cheap check first)
     std::unique_lock<std::mutex> lk(d->mu, std::try_to_lock);
@@ -786,6 +811,9 @@ DFCCL_API ncclResult_t ofcclInitRankCtx(ofcclRankCtx_t* rankCtx, int rank) {
   ofcclRankCtx* c = new ofcclRankCtx();
   c->rank = rank;
   c->device = device;
+  // QLen of the reference (src/include/collectives_ofccl.h:104,110); a smaller queue is only of use to tests of
+  // the full-queue path
+  c->sqCapacity = (uint64_t)std::min<int64_t>(kSqCapacity, std::max<int64_t>(1, envInt("DFCCL_SQ_CAPACITY", kSqCapacity)));
   for (int i = 0; i < kMaxColls; i++) {
     c->collIndex[i] = -1;
     c->callbacks[i] = nullptr;
@@ -910,6 +938,7 @@ DFCCL_API ncclResult_t ofcclFinalizeRankCtx7StartHostThrds(ofcclRankCtx_t c) {
     if (slot < 0) return ncclInvalidUsage;
     d->readKnobs();
     d->quiesceLocked(lk);
+    if (d->running) giveUpOnResidentDaemon(d, "attaching a rank context");
     d->slots[slot] = c;
     d->nActive++;
     c->slot = slot;
@@ -939,7 +968,9 @@ DFCCL_API ncclResult_t ofcclDestroy(ofcclRankCtx_t c) {
     Daemon* d = c->daemon;
     bool quitSent = false;
     bool lastRank = false;
-    const auto deadline = std::chrono::steady_clock::now() + std::chrono::seconds(20);
+    // (DFCCL_DESTROY_WAIT_MS: how long the rank's workgroups are given to leave; 20 s unless a test says otherwise)
+    const auto deadline = std::chrono::steady_clock::now() +
+                          std::chrono::milliseconds(std::max<int64_t>(1, envInt("DFCCL_DESTROY_WAIT_MS", 20000)));
     for (;;) {
       std::unique_lock<std::mutex> lk(d->mu);
       bool out = !d->running;
@@ -971,7 +1002,8 @@ DFCCL_API ncclResult_t ofcclDestroy(ofcclRankCtx_t c) {
         // an aborted kernel abandons its scheduler state: it must never be launched again on top of it
         d->failed = true;
         __atomic_store_n(d->ctrl, kCtrlAbort, __ATOMIC_RELEASE);
-        d->cv.wait_for(lk, std::chrono::seconds(10), [&] { return !d->running; });
+        d->cv.wait_for(lk, std::chrono::milliseconds(Daemon::abortWaitMs()), [&] { return !d->running; });
+        if (d->running) giveUpOnResidentDaemon(d, "destroying a rank context");
         d->slots[c->slot] = nullptr;
         d->nActive--;
         lastRank = (d->nActive == 0);
@@ -1083,6 +1115,7 @@ DFCCL_API ncclResult_t dfcclGetStats(ofcclRankCtx_t c, dfcclStats* out) {
     out->forcedQuits += __atomic_load_n(&s->forcedQuits, __ATOMIC_ACQUIRE);
     out->slicesMoved += __atomic_load_n(&s->slicesMoved, __ATOMIC_ACQUIRE);
   }
+  out->sqFullWaits = c->sqFullSpins.load(std::memory_order_relaxed);
   std::lock_guard<std::mutex> lk(d->mu);
   out->daemonLaunches = d->launches;
   return ncclSuccess;

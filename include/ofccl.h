@@ -124,11 +124,17 @@ ncclResult_t ofcclPrepareAllGather(size_t sendcount, ncclDataType_t datatype, nc
 
 /* ---- run: submit one instance of a prepared collective --------------------
  * Builds a submission-queue entry and spins while the queue is full
- * (src/collectives_ofccl/ofccl_all_reduce.cc:18-34); always returns
- * ncclSuccess once the entry is queued.  sendbuff / recvbuff are device
- * pointers that must stay valid until `callback(collId, callbackArgs)` has
- * been called on the poller thread.  At most one instance per collId may be
- * in flight; a second Run for the same collId waits for the first. */
+ * (src/collectives_ofccl/ofccl_all_reduce.cc:18-34).  Returns ncclSuccess once
+ * the entry is queued.  Unlike the reference, which always returns ncclSuccess
+ * (ofccl_all_reduce.cc:29-33), a Run returns ncclSystemError when the daemon
+ * kernel could not be launched or had to be aborted (also out of the wait for a
+ * full queue or for an earlier instance): no callback will come for that call.
+ * ncclInvalidUsage / ncclInvalidArgument report a context that is not
+ * finalized, an unknown collId or a pointer that is not a device address.
+ * sendbuff / recvbuff are device pointers that must stay valid until
+ * `callback(collId, callbackArgs)` has been called on the poller thread.  At
+ * most one instance per collId may be in flight; a second Run for the same
+ * collId waits for the first. */
 ncclResult_t ofcclRunReduce(const void* sendbuff, void* recvbuff, int collId, CallbackFunc callback,
                             void* callbackArgs, ofcclRankCtx_t rankCtx);                   /* nccl.h.in:256 */
 ncclResult_t ofcclRunBcast(void* buff, int collId, CallbackFunc callback, void* callbackArgs,
@@ -166,6 +172,7 @@ typedef struct {
   uint64_t daemonLaunches;  /* daemon kernel launches on this device         */
   uint64_t forcedQuits;     /* preemptions raised by DFCCL_FORCE_QUIT_EVERY  */
   uint64_t slicesMoved;     /* reduce-copy / copy slices executed            */
+  uint64_t sqFullWaits;     /* times a Run found the submission queue full and had to wait (host side) */
 } dfcclStats;
 
 /* Sums the counters over this rank's workgroups. Valid after Finalize; exact

@@ -43,6 +43,7 @@ static std::vector<std::shared_ptr<Job>>& gJobs = *new std::vector<std::shared_p
 static Stream& gNullStream = *new Stream();
 
 int gJitterPerMille = getenv("EMUL_JITTER") ? atoi(getenv("EMUL_JITTER")) : 0;
+bool gNeverLeave = getenv("EMUL_NEVER_LEAVE") && atoi(getenv("EMUL_NEVER_LEAVE")) != 0;
 void jitterSleep() {
   static thread_local uint64_t rng = 0x9e3779b97f4a7c15ull ^ ((uint64_t)tls.bIdx.x << 32) ^ tls.tIdx.x ^ (uint64_t)time(nullptr) << 16;
   rng ^= rng << 13;

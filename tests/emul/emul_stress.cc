@@ -4,12 +4,19 @@
 // data race in LDS (ThreadSanitizer build) ends the process with a report.
 //
 //   emul_stress repeat <ranks> <count> <reps> <colls>   the same small fp32 Sum all-reduces over and over, one
-//        after the other, every rank submitted in turn from this thread (the shape of the parked GPU test
-//        test_small_all_reduce_repeated_express_and_fallbacks); knobs come from the environment
+//        after the other, every rank submitted in turn from this thread (the shape of the GPU test
+//        test_small_all_reduce_repeated_and_fallbacks); knobs come from the environment
 //   emul_stress mixed <ranks> <reps>    all five collectives side by side, int32, ranks submit in different orders
 //   emul_stress relaunch <ranks>        idle exit and relaunch, with and without a collective parked
 //   emul_stress reuse <ranks>           rank contexts destroyed and created again: old communicators are refused
 //   emul_stress fuzz <seed> <rounds>    random collectives, ranks and submission orders
+//   emul_stress backpressure <ranks> <colls> <rounds> <callback sleep us>   two submitting threads per rank push
+//        every collective `rounds` times as fast as the queue takes them (DFCCL_SQ_CAPACITY makes it small), the
+//        last rank starting late; every submission must get exactly one callback
+//   emul_stress tworings <ranks>        one ring stays busy while the other's workgroups leave for idleness; the
+//        idle ring's next submission must still get through (the whole daemon leaves and is launched again)
+//   emul_stress stuck <ranks>           (with EMUL_NEVER_LEAVE=1) the daemon never leaves: Destroy must end the
+//        process with a report instead of blocking for good
 #include <hip/hip_runtime.h>
 #include <ofccl.h>
 #include <unistd.h>
@@ -106,7 +113,7 @@ static uint16_t bf16Of(int v) {  // small integers are exact in bfloat16
 
 // Collective 0 is an fp32 Sum of `count` elements; a second one, if asked for, a bf16 Max of 3 * count.  With two
 // the order is 0, 0, 1, 0, 0, 1, ...: the context that is resident in the workgroup changes now and then, and
-// every second run of collective 0 finds its context resident (the condition of the express path).
+// every second run of collective 0 finds its context resident.
 static int scenarioRepeat(int n, int count, int reps, int ncolls) {
   Ring ring(n);
   if (ncolls > 2) ncolls = 2;
@@ -448,6 +455,192 @@ static int scenarioFuzz(uint64_t seed, int rounds) {
   return 0;
 }
 
+// Back-pressure of the queues: `colls` small all-reduces, every rank has two threads that submit all of them
+// `rounds` times (a collective again as soon as its previous instance has called back), the last rank starts
+// 200 ms late so that the others pile up parked collectives, and the callback sleeps for `cbSleepUs` on the
+// poller thread.  Checks: every submission got exactly one callback, results are right, and (when the queue was
+// made small) the full-queue path was taken.
+static int scenarioBackpressure(int n, int ncolls, int rounds, int cbSleepUs) {
+  const int count = 600;
+  Ring ring(n);
+  for (int c = 0; c < ncolls; c++) {
+    auto& comms = ring.newComms();
+    for (int r = 0; r < n; r++) CHECK(ofcclPrepareAllReduce(count, ncclInt32, ncclSum, comms[r], c, ring.ctxs[r]));
+  }
+  ring.finalize();
+  struct CbArg { std::atomic<int> calls{0}; int sleepUs = 0; };
+  std::vector<CbArg> args((size_t)n * ncolls);
+  for (auto& a : args) a.sleepUs = cbSleepUs;
+  auto cb = +[](int, void* p) {
+    CbArg* a = (CbArg*)p;
+    if (a->sleepUs > 0) usleep((useconds_t)a->sleepUs);
+    a->calls.fetch_add(1);
+    return 0;
+  };
+  std::vector<std::vector<int32_t*>> send((size_t)ncolls), recv((size_t)ncolls);
+  for (int c = 0; c < ncolls; c++)
+    for (int r = 0; r < n; r++) {
+      send[c].push_back(devAlloc<int32_t>(count));
+      recv[c].push_back(devAlloc<int32_t>(count));
+      for (int i = 0; i < count; i++) {
+        send[c][r][i] = i + 3 * r + 7 * c;
+        recv[c][r][i] = -1;
+      }
+    }
+  std::atomic<int> failures{0};
+  std::vector<std::thread> threads;
+  for (int r = 0; r < n; r++)
+    for (int half = 0; half < 2; half++)
+      threads.emplace_back([&, r, half] {
+        if (r == n - 1) usleep(200000);
+        for (int round = 0; round < rounds; round++)
+          for (int c = half; c < ncolls; c += 2) {
+            CbArg& a = args[(size_t)r * ncolls + c];
+            // (a second Run of a collective waits for the first inside the library; the test adds no wait of its own)
+            const ncclResult_t res = ofcclRunAllReduce(send[c][r], recv[c][r], c, cb, &a, ring.ctxs[r]);
+            if (res != ncclSuccess) failures.fetch_add(1);
+          }
+      });
+  for (auto& t : threads) t.join();
+  const auto t0 = std::chrono::steady_clock::now();
+  for (;;) {
+    bool all = true;
+    for (auto& a : args) all = all && a.calls.load() >= rounds;
+    if (all) break;
+    if (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 240.0) {
+      fprintf(stderr, "emul_stress: backpressure: callbacks missing after 240 s\n");
+      dfcclDumpState(ring.ctxs[0]);
+      emulDumpThreads();
+      return 3;
+    }
+    usleep(1000);
+  }
+  usleep(50000);  // a callback too many would show up now
+  for (auto& a : args)
+    if (a.calls.load() != rounds) {
+      fprintf(stderr, "emul_stress: backpressure: %d callbacks for %d submissions\n", a.calls.load(), rounds);
+      return 1;
+    }
+  for (int c = 0; c < ncolls; c++)
+    for (int r = 0; r < n; r++)
+      for (int i = 0; i < count; i++) {
+        int32_t e = 0;
+        for (int q = 0; q < n; q++) e += i + 3 * q + 7 * c;
+        if (recv[c][r][i] != e) {
+          fprintf(stderr, "emul_stress: backpressure: collective %d rank %d element %d: %d, expected %d\n", c, r, i, recv[c][r][i], e);
+          return 1;
+        }
+      }
+  uint64_t fullWaits = 0, cqes = 0;
+  dfcclStats st;
+  for (int r = 0; r < n; r++) {
+    CHECK(dfcclGetStats(ring.ctxs[r], &st));
+    fullWaits += st.sqFullWaits;
+    cqes += st.cqesWritten;
+  }
+  ring.destroy();
+  freeBuffers();
+  if (failures.load() != 0 || cqes != (uint64_t)n * ncolls * rounds) {
+    fprintf(stderr, "emul_stress: backpressure: %d failed submissions, %llu completions\n", failures.load(), (unsigned long long)cqes);
+    return 1;
+  }
+  const char* cap = getenv("DFCCL_SQ_CAPACITY");
+  if (cap != nullptr && atoi(cap) < ncolls / 2 && fullWaits == 0) {
+    fprintf(stderr, "emul_stress: backpressure: the queue of %s entries was never found full\n", cap);
+    return 1;
+  }
+  printf("backpressure: %d ranks x %d collectives x %d rounds ok, %llu completions, queue found full %llu times\n", n,
+         ncolls, rounds, (unsigned long long)cqes, (unsigned long long)fullWaits);
+  return 0;
+}
+
+// Two rings on one daemon.  Ring A keeps running small all-reduces; ring B stays silent until its workgroups have
+// left for idleness (TOLERANT_UNPROGRESSED_CNT is small), then submits.  B's submission is only seen after a new
+// launch, which needs A's workgroups to leave too although they are busy.
+static int scenarioTwoRings(int n) {
+  const int count = 500;
+  Ring a(n), b(n);
+  auto& ca = a.newComms();
+  for (int r = 0; r < n; r++) CHECK(ofcclPrepareAllReduce(count, ncclInt32, ncclSum, ca[r], 0, a.ctxs[r]));
+  auto& cb = b.newComms();
+  for (int r = 0; r < n; r++) CHECK(ofcclPrepareAllReduce(count, ncclInt32, ncclSum, cb[r], 0, b.ctxs[r]));
+  a.finalize();
+  b.finalize();
+  std::vector<int32_t*> sa, ra, sb, rb;
+  for (int r = 0; r < n; r++) {
+    sa.push_back(devAlloc<int32_t>(count));
+    ra.push_back(devAlloc<int32_t>(count));
+    sb.push_back(devAlloc<int32_t>(count));
+    rb.push_back(devAlloc<int32_t>(count));
+    for (int i = 0; i < count; i++) {
+      sa[r][i] = i + r;
+      sb[r][i] = 5 * i - r;
+    }
+  }
+  std::atomic<bool> stop{false};
+  std::atomic<int> repsA{0};
+  std::thread busy([&] {
+    std::vector<int> want((size_t)n, 0);
+    while (!stop.load()) {
+      for (int r = 0; r < n; r++) {
+        want[r]++;
+        CHECK(ofcclRunAllReduce(sa[r], ra[r], 0, Ring::cb, &a.flag(r, 0), a.ctxs[r]));
+      }
+      a.waitAll(want, 180.0, "two rings, the busy ring");
+      repsA.fetch_add(1);
+    }
+  });
+  sleep(4);  // ring B's workgroups have seen nothing for long and have left
+  std::vector<int> wantB((size_t)n, 1);
+  for (int r = 0; r < n; r++) CHECK(ofcclRunAllReduce(sb[r], rb[r], 0, Ring::cb, &b.flag(r, 0), b.ctxs[r]));
+  b.waitAll(wantB, 120.0, "two rings, the ring that had gone idle");
+  stop.store(true);
+  busy.join();
+  for (int r = 0; r < n; r++)
+    for (int i = 0; i < count; i++) {
+      int32_t eb = 0, ea = 0;
+      for (int q = 0; q < n; q++) {
+        eb += 5 * i - q;
+        ea += i + q;
+      }
+      if (rb[r][i] != eb || ra[r][i] != ea) {
+        fprintf(stderr, "emul_stress: tworings: rank %d element %d: %d / %d, expected %d / %d\n", r, i, ra[r][i], rb[r][i], ea, eb);
+        return 1;
+      }
+    }
+  dfcclStats st;
+  CHECK(dfcclGetStats(b.ctxs[0], &st));
+  a.destroy();
+  b.destroy();
+  freeBuffers();
+  printf("tworings: ok, %d collectives of the busy ring, %llu daemon launches\n", repsA.load(), (unsigned long long)st.daemonLaunches);
+  return st.daemonLaunches >= 2 ? 0 : 1;
+}
+
+// With EMUL_NEVER_LEAVE=1 no workgroup ever leaves the kernel.  One collective runs, then Destroy: after its wait
+// (DFCCL_DESTROY_WAIT_MS) and the abort's (DFCCL_ABORT_WAIT_MS) the library has to report and end the process
+// with status 70; returning from Destroy, or blocking for good, is the failure.
+static int scenarioStuck(int n) {
+  const int count = 1000;
+  Ring ring(n);
+  auto& comms = ring.newComms();
+  for (int r = 0; r < n; r++) CHECK(ofcclPrepareAllReduce(count, ncclInt32, ncclSum, comms[r], 0, ring.ctxs[r]));
+  ring.finalize();
+  std::vector<int32_t*> send, recv;
+  for (int r = 0; r < n; r++) {
+    send.push_back(devAlloc<int32_t>(count));
+    recv.push_back(devAlloc<int32_t>(count));
+    for (int i = 0; i < count; i++) send[r][i] = i;
+  }
+  std::vector<int> want((size_t)n, 1);
+  for (int r = 0; r < n; r++) CHECK(ofcclRunAllReduce(send[r], recv[r], 0, Ring::cb, &ring.flag(r, 0), ring.ctxs[r]));
+  ring.waitAll(want, 120.0, "stuck");
+  printf("stuck: collective done, destroying\n");
+  ofcclDestroy(ring.ctxs[0]);
+  printf("stuck: ofcclDestroy returned although the daemon cannot have left\n");
+  return 1;
+}
+
 int main(int argc, char** argv) {
   setvbuf(stdout, nullptr, _IOLBF, 0);
   setenv("DFCCL_STATS_WAIT_MS", "5000", 0);  // emulated workgroups answer a request for their counters slowly
@@ -457,6 +650,9 @@ int main(int argc, char** argv) {
   if (mode == "relaunch" && argc == 3) return scenarioRelaunch(atoi(argv[2]));
   if (mode == "reuse" && argc == 3) return scenarioReuse(atoi(argv[2]));
   if (mode == "fuzz" && argc == 4) return scenarioFuzz(strtoull(argv[2], nullptr, 10), atoi(argv[3]));
+  if (mode == "backpressure" && argc == 6) return scenarioBackpressure(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]));
+  if (mode == "tworings" && argc == 3) return scenarioTwoRings(atoi(argv[2]));
+  if (mode == "stuck" && argc == 3) return scenarioStuck(atoi(argv[2]));
   fprintf(stderr, "usage: emul_stress repeat <ranks> <count> <reps> <colls> | mixed <ranks> <reps> | relaunch <ranks> | reuse <ranks> | fuzz <seed> <rounds>\n");
   return 64;
 }

@@ -152,6 +152,10 @@ void launch(Stream* s, unsigned grid, unsigned block, std::function<void()> body
 
 #define DFCCL_WAVE_UNIFORM(x) ::emul::shflFrom((x), 0, __LINE__)
 
+// EMUL_NEVER_LEAVE=1: the daemon's workgroups ignore every reason to leave (see DFCCL_TEST_NEVER_LEAVES in daemon.hip)
+namespace emul { extern bool gNeverLeave; }
+#define DFCCL_TEST_NEVER_LEAVES() (::emul::gNeverLeave)
+
 // the one LDS object of the daemon kernel
 #define DFCCL_WG_SHARED(T, name) T& name = *reinterpret_cast<T*>(::emul::wgSharedMem(sizeof(T)))
 
@@ -168,6 +172,7 @@ typedef ::emul::Dim3 dim3;
 
 // ---- compiler builtins of the target
 #define __builtin_amdgcn_readfirstlane(x) (x)  // only ever applied to values that are the same in every lane
+#define __builtin_amdgcn_readlane(x, srcLane) ::emul::shflFrom((x), (srcLane), __LINE__)
 #define __builtin_amdgcn_fence(order, scope) __atomic_thread_fence(__ATOMIC_SEQ_CST)
 #define __builtin_amdgcn_s_sleep(n) sched_yield()
 #define __HIP_MEMORY_SCOPE_AGENT 0

@@ -47,11 +47,11 @@ def no_sanitizer_report(r):
 TINY = {"BASE_CTX_SWITCH_THRESHOLD": "1", "NUM_TRY_TASKQ_HEAD": "1", "RECV_SUCCESS_FACTOR": "0"}
 
 SCENARIOS = [
-    # the same small all-reduces over and over, ranks submitted in turn: scheduler path, then wave 0's express
-    # path, then the express path with every bounded wait giving up after one look
+    # the same small all-reduces over and over, ranks submitted in turn (one tile per rank: wave 0 runs them
+    # alone), then with every bounded wait giving up after one look, then too large for a wave on its own
     ("repeat-default", {}, ["repeat", "4", "2048", "12", "2"]),
-    ("repeat-express", {"DFCCL_EXPRESS": "1"}, ["repeat", "4", "2048", "12", "2"]),
-    ("repeat-express-tiny-budget", dict(TINY, DFCCL_EXPRESS="1"), ["repeat", "4", "2048", "20", "2"]),
+    ("repeat-tiny-budget", TINY, ["repeat", "4", "2048", "20", "2"]),
+    ("repeat-whole-workgroup", {}, ["repeat", "4", "6000", "8", "2"]),
     ("repeat-tiny-budget-ragged", TINY, ["repeat", "3", "5000", "6", "2"]),
     ("repeat-8-ranks", {}, ["repeat", "8", "2048", "4", "1"]),
     ("repeat-several-channels", {"NCCL_MAX_NCHANNELS": "8"}, ["repeat", "2", "300000", "2", "1"]),
@@ -68,21 +68,30 @@ SCENARIOS = [
     # a daemon that leaves every 50 ms, whatever it is doing, and is launched again: state saved and restored
     ("short-lifetime-direct", {"DFCCL_DAEMON_MAX_MS": "50"}, ["mixed", "4", "2"]),
     ("short-lifetime-fifo", {"DFCCL_DAEMON_MAX_MS": "50", "DFCCL_PROTO": "fifo"}, ["mixed", "3", "2"]),
-    ("short-lifetime-express", {"DFCCL_DAEMON_MAX_MS": "50", "DFCCL_EXPRESS": "1"}, ["repeat", "4", "2048", "20", "2"]),
+    ("short-lifetime-small", {"DFCCL_DAEMON_MAX_MS": "50"}, ["repeat", "4", "2048", "20", "2"]),
     # random ranks, collectives, sizes, roots and submission orders (three rounds each)
     ("random-direct", {"NCCL_MAX_NCHANNELS": "2"}, ["fuzz", "1003", "3"]),
     ("random-fifo-short-lifetime", {"NCCL_MAX_NCHANNELS": "2", "DFCCL_PROTO": "fifo", "DFCCL_DAEMON_MAX_MS": "57"},
      ["fuzz", "1007", "3"]),
-    ("random-express-tiny-budget", dict(TINY, NCCL_MAX_NCHANNELS="2", DFCCL_EXPRESS="1"), ["fuzz", "1012", "3"]),
+    ("random-tiny-budget", dict(TINY, NCCL_MAX_NCHANNELS="2"), ["fuzz", "1012", "3"]),
     # rank contexts destroyed and created again on the same daemon; a communicator that has run is refused
     ("reuse", {}, ["reuse", "3"]),
+    # the queues' back-pressure: a submission queue of 4 entries under two submitting threads per rank and a late
+    # rank (the full-queue path and the lazily published head), then the full-size queue with a callback that
+    # sleeps 2 ms on the poller thread; every submission gets exactly one callback
+    ("backpressure-small-queue", {"DFCCL_SQ_CAPACITY": "4"}, ["backpressure", "3", "24", "3", "0"]),
+    ("backpressure-small-queue-channels", {"DFCCL_SQ_CAPACITY": "3", "NCCL_MAX_NCHANNELS": "2",
+                                           "DFCCL_BYTES_PER_CHANNEL": "512"}, ["backpressure", "2", "16", "3", "0"]),
+    ("backpressure-slow-callback", {}, ["backpressure", "2", "40", "2", "2000"]),
+    # one ring busy, the other's workgroups gone for idleness: its next submission still gets through
+    ("two-rings-idle-exit", {"TOLERANT_UNPROGRESSED_CNT": "300"}, ["tworings", "2"]),
 ]
 
 
 @pytest.mark.parametrize("name,env,args", SCENARIOS, ids=[s[0] for s in SCENARIOS])
 def test_emulated_daemon(stress, name, env, args):
     e = dict(os.environ)
-    for k in ("DFCCL_PROTO", "DFCCL_EXPRESS", "DFCCL_FORCE_QUIT_EVERY", "BASE_CTX_SWITCH_THRESHOLD"):
+    for k in ("DFCCL_PROTO", "DFCCL_FORCE_QUIT_EVERY", "BASE_CTX_SWITCH_THRESHOLD"):
         e.pop(k, None)
     e.update({"EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "120", "DFCCL_DAEMON_MAX_MS": "100000"})
     e.update(env)
@@ -90,6 +99,20 @@ def test_emulated_daemon(stress, name, env, args):
     assert r.returncode == 0, f"{name}: rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
     assert " ok" in r.stdout
     assert no_sanitizer_report(r), r.stderr[-6000:]
+
+
+def test_a_daemon_that_never_leaves_ends_the_process_with_a_report(stress):
+    # the workgroups ignore every reason to leave (a host-side stand-in for a workgroup stuck at a barrier):
+    # Destroy waits, aborts, waits again, then prints what it knows and ends the process instead of joining a
+    # thread that waits for the kernel and freeing memory the kernel still uses
+    e = dict(os.environ)
+    e.update({"EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "120", "EMUL_NEVER_LEAVE": "1", "DFCCL_DESTROY_WAIT_MS": "1500",
+              "DFCCL_ABORT_WAIT_MS": "1500"})
+    r = subprocess.run([stress, "stuck", "2"], env=sanitizer_env(e, leaks=False), capture_output=True, text=True,
+                       timeout=120 * SLOW)
+    assert r.returncode == 70, f"rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
+    assert "still resident after an abort request" in r.stderr
+    assert "ofcclDestroy returned" not in r.stdout
 
 
 DRIVER = [

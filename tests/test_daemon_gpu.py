@@ -477,18 +477,13 @@ def test_other_collectives_disordered_submission(proto):
                 assert np.array_equal(to_np(orc.F32, bufs[cid][1][r]), wants[cid][r]), (cid, kind, r)
 
 
-@pytest.mark.skipif(os.environ.get("DFCCL_RUN_PARKED") != "1",
-                    reason="both GPU runs that included this test lost their box (a wave's lanes read a flag in LDS "
-                           "before lane 0 had written it; fixed since, passes on the host emulation); its one "
-                           "confirming run on a GPU is still to come (DFCCL_RUN_PARKED=1 runs it)")
-@pytest.mark.parametrize("knobs", [{"DFCCL_EXPRESS": "1", "BASE_CTX_SWITCH_THRESHOLD": "1", "NUM_TRY_TASKQ_HEAD": "1",
-                                    "RECV_SUCCESS_FACTOR": "0"},
-                                   {"DFCCL_EXPRESS": "0"}, {"DFCCL_EXPRESS": "1", "DFCCL_IDLE_POLL_ROUNDS": "0"},
-                                   {"DFCCL_EXPRESS": "1"}])
-def test_small_all_reduce_repeated_express_and_fallbacks(knobs, monkeypatch):
-    # the same small collective over and over (its context stays resident, so wave 0 runs it on the spot); with a
-    # spin budget of one poll most of those attempts run out at one of the two waits and hand over to the
-    # scheduler, because the ranks are submitted one after the other from this thread
+@pytest.mark.parametrize("knobs", [{"BASE_CTX_SWITCH_THRESHOLD": "1", "NUM_TRY_TASKQ_HEAD": "1", "RECV_SUCCESS_FACTOR": "0"},
+                                   {}, {"DFCCL_IDLE_POLL_ROUNDS": "0"}])
+def test_small_all_reduce_repeated_and_fallbacks(knobs, monkeypatch):
+    # the same small collectives over and over: each rank's share is one tile of 2 KiB / 3 KiB, which wave 0 of the
+    # workgroup runs on its own (waits, fold, release, final wait without a workgroup barrier in between); with a
+    # spin budget of one poll most visits run out at one of the two waits and park the collective, because the
+    # ranks are submitted one after the other from this thread
     from dfccl_amd.ring import VirtualRing
     for k, v in knobs.items():
         monkeypatch.setenv(k, v)
