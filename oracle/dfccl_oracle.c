@@ -9,14 +9,15 @@
 
 int orc_type_size(int dtype) {
   switch (dtype) {
-    case ORC_I8: return 1;
-    case ORC_I32: return 4;
-    case ORC_F16: return 2;
-    case ORC_F32: return 4;
-    case ORC_BF16: return 2;
+    case ORC_I8: case ORC_U8: return 1;
+    case ORC_I32: case ORC_U32: case ORC_F32: return 4;
+    case ORC_I64: case ORC_U64: case ORC_F64: return 8;
+    case ORC_F16: case ORC_BF16: return 2;
     default: return 0;
   }
 }
+
+static int is_float_type(int dtype) { return dtype == ORC_F16 || dtype == ORC_BF16 || dtype == ORC_F32 || dtype == ORC_F64; }
 
 /* ---------------------------------------------------------------- soft float */
 
@@ -105,6 +106,48 @@ static inline int8_t op_i8(int op, int8_t a, int8_t b) {
     default: return (a < b) ? a : b;
   }
 }
+/* the generic functors of src/include/reduce_kernel.h:23-53 on the remaining integer types (unsigned arithmetic
+ * wraps; Max = (x<y)?y:x, Min = (x<y)?x:y) and fmax / fmin for double (:456-469) */
+static inline uint8_t op_u8(int op, uint8_t a, uint8_t b) {
+  switch (op) {
+    case ORC_SUM: return (uint8_t)(a + b);
+    case ORC_PROD: return (uint8_t)((unsigned)a * (unsigned)b);
+    case ORC_MAX: return (a > b) ? a : b;
+    default: return (a < b) ? a : b;
+  }
+}
+static inline uint32_t op_u32(int op, uint32_t a, uint32_t b) {
+  switch (op) {
+    case ORC_SUM: return a + b;
+    case ORC_PROD: return a * b;
+    case ORC_MAX: return (a < b) ? b : a;
+    default: return (a < b) ? a : b;
+  }
+}
+static inline int64_t op_i64(int op, int64_t a, int64_t b) {
+  switch (op) {
+    case ORC_SUM: return (int64_t)((uint64_t)a + (uint64_t)b);
+    case ORC_PROD: return (int64_t)((uint64_t)a * (uint64_t)b);
+    case ORC_MAX: return (a < b) ? b : a;
+    default: return (a < b) ? a : b;
+  }
+}
+static inline uint64_t op_u64(int op, uint64_t a, uint64_t b) {
+  switch (op) {
+    case ORC_SUM: return a + b;
+    case ORC_PROD: return a * b;
+    case ORC_MAX: return (a < b) ? b : a;
+    default: return (a < b) ? a : b;
+  }
+}
+static inline double op_f64(int op, double a, double b) {
+  switch (op) {
+    case ORC_SUM: return a + b;
+    case ORC_PROD: return a * b;
+    case ORC_MAX: return fmax(a, b);
+    default: return fmin(a, b);
+  }
+}
 static inline uint16_t op_f16(int op, uint16_t a, uint16_t b) {
   return orc_f32_to_f16(op_f32(op, orc_f16_to_f32(a), orc_f16_to_f32(b)));
 }
@@ -119,6 +162,11 @@ void orc_apply(int dtype, int op, const void* a, const void* b, void* out) {
     case ORC_F16: *(uint16_t*)out = op_f16(op, *(const uint16_t*)a, *(const uint16_t*)b); break;
     case ORC_F32: *(float*)out = op_f32(op, *(const float*)a, *(const float*)b); break;
     case ORC_BF16: *(uint16_t*)out = op_bf16(op, *(const uint16_t*)a, *(const uint16_t*)b); break;
+    case ORC_U8: *(uint8_t*)out = op_u8(op, *(const uint8_t*)a, *(const uint8_t*)b); break;
+    case ORC_U32: *(uint32_t*)out = op_u32(op, *(const uint32_t*)a, *(const uint32_t*)b); break;
+    case ORC_I64: *(int64_t*)out = op_i64(op, *(const int64_t*)a, *(const int64_t*)b); break;
+    case ORC_U64: *(uint64_t*)out = op_u64(op, *(const uint64_t*)a, *(const uint64_t*)b); break;
+    case ORC_F64: *(double*)out = op_f64(op, *(const double*)a, *(const double*)b); break;
     default: break;
   }
 }
@@ -142,32 +190,127 @@ static void apply_range(int dtype, int op, const void* a, const void* b, void* o
     case ORC_F16: RANGE_LOOP(uint16_t, op_f16); break;
     case ORC_F32: RANGE_LOOP(float, op_f32); break;
     case ORC_BF16: RANGE_LOOP(uint16_t, op_bf16); break;
+    case ORC_U8: RANGE_LOOP(uint8_t, op_u8); break;
+    case ORC_U32: RANGE_LOOP(uint32_t, op_u32); break;
+    case ORC_I64: RANGE_LOOP(int64_t, op_i64); break;
+    case ORC_U64: RANGE_LOOP(uint64_t, op_u64); break;
+    case ORC_F64: RANGE_LOOP(double, op_f64); break;
     default: break;
   }
 }
 
+/* ------------------------------------------------- scaled sums (ncclAvg, PreMulSum)
+ *
+ * The reference turns ncclAvg into a device op with a scalar (hostToDevRedOp, src/enqueue.cc:1305-1371):
+ * integer types -> SumPostDiv with n = nRanks, float types -> PreMulSum with the scalar 1/nRanks converted
+ * to the element type.  PreMulSum multiplies every rank's input by the scalar as it enters the reduction
+ * (preOp on the user-input source, src/collectives_ofccl/device/ofccl_prims_simple.h:405-411,
+ * src/include/common_kernel.h:506-538), one correctly rounded multiply in the element type
+ * (src/include/reduce_kernel.h:503-668); SumPostDiv divides the finished sum, T(x / n) with C++ integer
+ * division (:491-501), at the step that writes the final value (postOp = true:
+ * ofccl_all_reduce.h:132, ofccl_reduce_scatter.h:84, ofccl_reduce.h:78). */
+
+typedef struct {
+  int base;      /* ORC_SUM..ORC_MIN: the op applied between elements */
+  int pre;       /* multiply every input by `scalar` (bits of one element) first */
+  int post;      /* divide the final value by (int)scalar */
+  uint64_t scalar;
+} orc_xop;
+
+uint64_t orc_avg_scalar(int dtype, int n) {
+  uint64_t bits = 0;
+  if (!is_float_type(dtype)) return (uint64_t)n;
+  if (dtype == ORC_F64) { double d = 1.0 / n; memcpy(&bits, &d, 8); }
+  else {
+    float f = (float)(1.0 / n);
+    if (dtype == ORC_F32) { uint32_t u = f2u(f); bits = u; }
+    else if (dtype == ORC_F16) bits = orc_f32_to_f16(f);
+    else bits = orc_f32_to_bf16(f);
+  }
+  return bits;
+}
+
+/* resolves a public op code (+ scalar for ORC_PREMULSUM, group size for ORC_AVG); returns 0 if valid */
+static int resolve_op(int dtype, int op, uint64_t scalar, int n, orc_xop* x) {
+  x->base = op; x->pre = 0; x->post = 0; x->scalar = 0;
+  if (op >= ORC_SUM && op <= ORC_MIN) return 0;
+  x->base = ORC_SUM;
+  if (op == ORC_AVG) {
+    x->scalar = orc_avg_scalar(dtype, n);
+    if (is_float_type(dtype)) x->pre = 1; else x->post = 1;
+    return 0;
+  }
+  if (op == ORC_PREMULSUM) { x->pre = 1; x->scalar = scalar; return 0; }
+  return -1;
+}
+
+/* out[i] = in[i] * scalar, one multiply in the element type */
+static void premul_range(int dtype, uint64_t scalar, const void* in, void* out, size_t n) {
+  const size_t s = (size_t)orc_type_size(dtype);
+  char k[8];
+  memcpy(k, &scalar, 8);  /* little endian: the low bytes hold the element */
+  for (size_t i = 0; i < n; i++) orc_apply(dtype, ORC_PROD, (const char*)in + i * s, k, (char*)out + i * s);
+}
+
+/* x[i] = T(x[i] / n), the integer division of C++ after the usual arithmetic conversions with `int n` */
+static void postdiv_range(int dtype, uint64_t scalar, void* x, size_t n) {
+  const int d = (int)scalar;
+  switch (dtype) {
+    case ORC_I8: { int8_t* p = x; for (size_t i = 0; i < n; i++) p[i] = (int8_t)((int)p[i] / d); break; }
+    case ORC_U8: { uint8_t* p = x; for (size_t i = 0; i < n; i++) p[i] = (uint8_t)((int)p[i] / d); break; }
+    case ORC_I32: { int32_t* p = x; for (size_t i = 0; i < n; i++) p[i] = p[i] / d; break; }
+    case ORC_U32: { uint32_t* p = x; for (size_t i = 0; i < n; i++) p[i] = p[i] / (uint32_t)d; break; }
+    case ORC_I64: { int64_t* p = x; for (size_t i = 0; i < n; i++) p[i] = p[i] / (int64_t)d; break; }
+    case ORC_U64: { uint64_t* p = x; for (size_t i = 0; i < n; i++) p[i] = p[i] / (uint64_t)(int64_t)d; break; }
+    default: break;
+  }
+}
+
+/* a rank's input as it enters the reduction: the buffer itself, or a scaled copy in tmp */
+static const void* entering(int dtype, const orc_xop* x, const void* in, void* tmp, size_t n) {
+  if (!x->pre) return in;
+  premul_range(dtype, x->scalar, in, tmp, n);
+  return tmp;
+}
+
 /* ------------------------------------------------------------- reduce-copy */
 
-static void reduce_copy_range(int dtype, int op, int k, const void* const* srcs, void* dst, size_t begin, size_t n) {
+static void reduce_copy_range(int dtype, const orc_xop* x, int k, const void* const* srcs, void* dst, size_t begin,
+                              size_t n) {
   size_t s = (size_t)orc_type_size(dtype);
   char* d = (char*)dst + begin * s;
-  if (k == 1) {
+  if (k == 1 && !x->pre && !x->post) {
     memmove(d, (const char*)srcs[0] + begin * s, n * s);
     return;
   }
-  /* fold left to right; the first op reads src0 and src1, later ones the running value */
-  apply_range(dtype, op, (const char*)srcs[0] + begin * s, (const char*)srcs[1] + begin * s, d, n);
-  for (int j = 2; j < k; j++) apply_range(dtype, op, d, (const char*)srcs[j] + begin * s, d, n);
+  /* fold left to right; the first op reads src0 and src1, later ones the running value.  Every source is a
+   * user input here, so a pre-multiplication applies to each of them. */
+  void* tmp = x->pre ? malloc(n * s + 1) : NULL;
+  void* tmp0 = x->pre ? malloc(n * s + 1) : NULL;
+  const void* first = entering(dtype, x, (const char*)srcs[0] + begin * s, tmp0, n);
+  if (k == 1) memmove(d, first, n * s);
+  else apply_range(dtype, x->base, first, entering(dtype, x, (const char*)srcs[1] + begin * s, tmp, n), d, n);
+  for (int j = 2; j < k; j++)
+    apply_range(dtype, x->base, d, entering(dtype, x, (const char*)srcs[j] + begin * s, tmp, n), d, n);
+  if (x->post) postdiv_range(dtype, x->scalar, d, n);
+  free(tmp);
+  free(tmp0);
 }
 
-int orc_reduce_copy(int dtype, int op, int k, const void* const* srcs, void* dst, size_t n) {
-  if (orc_type_size(dtype) == 0 || k < 1 || op < 0 || op > 3) return -1;
-  reduce_copy_range(dtype, op, k, srcs, dst, 0, n);
+int orc_reduce_copy_x(int dtype, int op, uint64_t scalar, int k, const void* const* srcs, void* dst, size_t n) {
+  orc_xop x;
+  if (orc_type_size(dtype) == 0 || k < 1 || resolve_op(dtype, op, scalar, k, &x) != 0) return -1;
+  reduce_copy_range(dtype, &x, k, srcs, dst, 0, n);
   return 0;
 }
 
+int orc_reduce_copy(int dtype, int op, int k, const void* const* srcs, void* dst, size_t n) {
+  return orc_reduce_copy_x(dtype, op, 0, k, srcs, dst, n);
+}
+
 typedef struct {
-  int dtype, op, k;
+  int dtype, k;
+  orc_xop x;
   const void* const* srcs;
   void* dst;
   size_t begin, n;
@@ -175,12 +318,13 @@ typedef struct {
 
 static void* rc_thread(void* p) {
   rc_job* j = (rc_job*)p;
-  reduce_copy_range(j->dtype, j->op, j->k, j->srcs, j->dst, j->begin, j->n);
+  reduce_copy_range(j->dtype, &j->x, j->k, j->srcs, j->dst, j->begin, j->n);
   return NULL;
 }
 
 int orc_reduce_copy_mt(int dtype, int op, int k, const void* const* srcs, void* dst, size_t n, int nthreads) {
-  if (orc_type_size(dtype) == 0 || k < 1 || op < 0 || op > 3) return -1;
+  orc_xop x;
+  if (orc_type_size(dtype) == 0 || k < 1 || resolve_op(dtype, op, 0, k, &x) != 0) return -1;
   if (nthreads <= 1) return orc_reduce_copy(dtype, op, k, srcs, dst, n);
   if (nthreads > 256) nthreads = 256;
   pthread_t th[256];
@@ -192,7 +336,7 @@ int orc_reduce_copy_mt(int dtype, int op, int k, const void* const* srcs, void* 
     size_t b = (size_t)t * per;
     if (b >= n) break;
     size_t len = (n - b < per) ? n - b : per;
-    jobs[t] = (rc_job){dtype, op, k, srcs, dst, b, len};
+    jobs[t] = (rc_job){dtype, k, x, srcs, dst, b, len};
     if (pthread_create(&th[t], NULL, rc_thread, &jobs[t]) != 0) {
       rc_thread(&jobs[t]);
       th[t] = 0;
@@ -232,10 +376,22 @@ static void local_copy(int dtype, const void* src, void* dst, int64_t n) {
 }
 
 int orc_all_reduce(int dtype, int op, const orc_geom* g, int64_t count, const void* const* send, void* const* recv) {
-  if (!geom_ok(g) || orc_type_size(dtype) == 0) return -1;
+  return orc_all_reduce_x(dtype, op, 0, g, count, send, recv);
+}
+
+int orc_all_reduce_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t count, const void* const* send,
+                     void* const* recv) {
+  orc_xop x;
+  if (!geom_ok(g) || orc_type_size(dtype) == 0 || resolve_op(dtype, op, scalar, g->n_ranks, &x) != 0) return -1;
   const int n = g->n_ranks;
   const size_t s = (size_t)orc_type_size(dtype);
-  if (n == 1) { local_copy(dtype, send[0], recv[0], count); return 0; }
+  if (n == 1) { /* one rank: a copy, with the scaling a sum of one term still gets */
+    const void* src[1] = {send[0]};
+    reduce_copy_range(dtype, &x, 1, src, recv[0], 0, (size_t)count);
+    return 0;
+  }
+  op = x.base;
+  char* tmp = malloc((size_t)round_up(g->chunk_elems, g->align_elems) * s + 1);
   const int64_t loop_size = (int64_t)g->n_channels * n * g->chunk_elems;
   const int64_t max_chunk = round_up(g->chunk_elems, g->align_elems);
   orc_msg* cur = calloc((size_t)n, sizeof(orc_msg));
@@ -261,12 +417,14 @@ int orc_all_reduce(int dtype, int op, const orc_geom* g, int64_t count, const vo
           if (nelem < 0) nelem = 0;
           const char* in = (const char*)send[r] + (size_t)off * s;
           char* out = (char*)recv[r] + (size_t)off * s;
+          if (step <= n - 1) in = entering(dtype, &x, in, tmp, (size_t)nelem); /* the steps that read the user's input */
           if (step == 0) { /* send */
             memcpy(cur[r].data, in, (size_t)nelem * s);
           } else if (step <= n - 2) { /* recvReduceSend */
             apply_range(dtype, op, in, prv[prev].data, cur[r].data, (size_t)nelem);
-          } else if (step == n - 1) { /* recvReduceCopySend */
+          } else if (step == n - 1) { /* recvReduceCopySend, postOp = true */
             apply_range(dtype, op, in, prv[prev].data, cur[r].data, (size_t)nelem);
+            if (x.post) postdiv_range(dtype, x.scalar, cur[r].data, (size_t)nelem);
             memcpy(out, cur[r].data, (size_t)nelem * s);
           } else if (step <= 2 * n - 3) { /* recvCopySend */
             memcpy(cur[r].data, prv[prev].data, (size_t)nelem * s);
@@ -281,7 +439,7 @@ int orc_all_reduce(int dtype, int op, const orc_geom* g, int64_t count, const vo
     }
   }
   for (int r = 0; r < n; r++) { free(cur[r].data); free(prv[r].data); }
-  free(cur); free(prv);
+  free(cur); free(prv); free(tmp);
   return 0;
 }
 
@@ -298,10 +456,22 @@ int orc_all_reduce_owner(const orc_geom* g, int64_t count, int64_t i) {
 
 int orc_reduce_scatter(int dtype, int op, const orc_geom* g, int64_t recvcount, const void* const* send,
                        void* const* recv) {
-  if (!geom_ok(g) || orc_type_size(dtype) == 0) return -1;
+  return orc_reduce_scatter_x(dtype, op, 0, g, recvcount, send, recv);
+}
+
+int orc_reduce_scatter_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t recvcount,
+                         const void* const* send, void* const* recv) {
+  orc_xop x;
+  if (!geom_ok(g) || orc_type_size(dtype) == 0 || resolve_op(dtype, op, scalar, g->n_ranks, &x) != 0) return -1;
   const int n = g->n_ranks;
   const size_t s = (size_t)orc_type_size(dtype);
-  if (n == 1) { local_copy(dtype, send[0], recv[0], recvcount); return 0; }
+  if (n == 1) {
+    const void* src[1] = {send[0]};
+    reduce_copy_range(dtype, &x, 1, src, recv[0], 0, (size_t)recvcount);
+    return 0;
+  }
+  op = x.base;
+  char* tmp = malloc((size_t)round_up(g->chunk_elems, g->align_elems) * s + 1);
   const int64_t loop_size = (int64_t)g->n_channels * g->chunk_elems;
   const int64_t max_chunk = round_up(g->chunk_elems, g->align_elems);
   orc_msg* cur = calloc((size_t)n, sizeof(orc_msg));
@@ -325,14 +495,15 @@ int orc_reduce_scatter(int dtype, int op, const orc_geom* g, int64_t recvcount, 
           else if (step <= n - 2) dest = (r + n - (step + 1)) % n;
           else dest = r;
           const int64_t off = chunk_off + (int64_t)dest * recvcount;
-          const char* in = (const char*)send[r] + (size_t)off * s;
+          const char* in = entering(dtype, &x, (const char*)send[r] + (size_t)off * s, tmp, (size_t)nelem);
           if (step == 0) {
             memcpy(cur[r].data, in, (size_t)nelem * s);
           } else if (step <= n - 2) {
             apply_range(dtype, op, in, prv[prev].data, cur[r].data, (size_t)nelem);
           } else {
-            /* stage through the message buffer so an in-place recv buffer is safe */
+            /* stage through the message buffer so an in-place recv buffer is safe; postOp = true */
             apply_range(dtype, op, in, prv[prev].data, cur[r].data, (size_t)nelem);
+            if (x.post) postdiv_range(dtype, x.scalar, cur[r].data, (size_t)nelem);
             memcpy((char*)recv[r] + (size_t)chunk_off * s, cur[r].data, (size_t)nelem * s);
           }
         }
@@ -341,7 +512,7 @@ int orc_reduce_scatter(int dtype, int op, const orc_geom* g, int64_t recvcount, 
     }
   }
   for (int r = 0; r < n; r++) { free(cur[r].data); free(prv[r].data); }
-  free(cur); free(prv);
+  free(cur); free(prv); free(tmp);
   return 0;
 }
 
@@ -396,11 +567,23 @@ int orc_all_gather(int dtype, const orc_geom* g, int64_t sendcount, const void* 
 
 int orc_reduce(int dtype, int op, const orc_geom* g, int64_t count, int root, const void* const* send,
                void* const* recv) {
-  if (!geom_ok(g) || orc_type_size(dtype) == 0) return -1;
+  return orc_reduce_x(dtype, op, 0, g, count, root, send, recv);
+}
+
+int orc_reduce_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t count, int root,
+                 const void* const* send, void* const* recv) {
+  orc_xop x;
+  if (!geom_ok(g) || orc_type_size(dtype) == 0 || resolve_op(dtype, op, scalar, g->n_ranks, &x) != 0) return -1;
   const int n = g->n_ranks;
   if (root < 0 || root >= n) return -1;
   const size_t s = (size_t)orc_type_size(dtype);
-  if (n == 1) { local_copy(dtype, send[0], recv[0], count); return 0; }
+  if (n == 1) {
+    const void* src[1] = {send[0]};
+    reduce_copy_range(dtype, &x, 1, src, recv[0], 0, (size_t)count);
+    return 0;
+  }
+  op = x.base;
+  char* tmp = malloc((size_t)round_up(g->chunk_elems, g->align_elems) * s + 1);
   const int64_t loop_size = (int64_t)g->n_channels * g->chunk_elems;
   const int64_t max_chunk = round_up(g->chunk_elems, g->align_elems);
   char* msg = malloc((size_t)max_chunk * s);
@@ -413,19 +596,21 @@ int orc_reduce(int dtype, int op, const orc_geom* g, int64_t count, int root, co
       /* the chain starts at the rank whose predecessor is the root and ends at the root */
       for (int k = 1; k <= n; k++) {
         const int r = (root + k) % n;
-        const char* in = (const char*)send[r] + (size_t)off * s;
+        const char* in = entering(dtype, &x, (const char*)send[r] + (size_t)off * s, tmp, (size_t)nelem);
         if (k == 1) {
           memcpy(msg, in, (size_t)nelem * s); /* send */
         } else if (k < n) {
           apply_range(dtype, op, in, msg, msg, (size_t)nelem); /* recvReduceSend */
         } else {
-          apply_range(dtype, op, in, msg, msg, (size_t)nelem); /* recvReduceCopy */
+          apply_range(dtype, op, in, msg, msg, (size_t)nelem); /* recvReduceCopy, postOp = true */
+          if (x.post) postdiv_range(dtype, x.scalar, msg, (size_t)nelem);
           memcpy((char*)recv[r] + (size_t)off * s, msg, (size_t)nelem * s);
         }
       }
     }
   }
   free(msg);
+  free(tmp);
   return 0;
 }
 

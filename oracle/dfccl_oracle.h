@@ -7,7 +7,9 @@
  *
  * What each function follows in the reference (paths relative to the reference
  * tree):
- *   element ops          src/include/reduce_kernel.h:23-53 (generic Sum/Prod/Max/Min),
+ *   element ops          src/include/reduce_kernel.h:23-53 (generic Sum/Prod/Max/Min, also for uint8 / uint32 /
+ *                        int64 / uint64), :456-469 (fp64 Max/Min = fmax/fmin),
+ *                        :485-704 (SumPostDiv, PreMulSum) with src/enqueue.cc:1305-1371 (what ncclAvg becomes),
  *                        :66-134 (int8 Sum/Prod wrap), :146-218 (int8 Max/Min signed),
  *                        :244-440 (fp16 / bf16: one correctly rounded op per step),
  *                        :442-455 (fp32 Max/Min = fmaxf/fminf)
@@ -45,8 +47,12 @@ extern "C" {
 
 /* dtype / op codes are the reference's ncclDataType_t / ncclRedOp_t values
  * (src/nccl.h.in:113-146). */
-enum { ORC_I8 = 0, ORC_I32 = 2, ORC_F16 = 6, ORC_F32 = 7, ORC_BF16 = 9 };
-enum { ORC_SUM = 0, ORC_PROD = 1, ORC_MAX = 2, ORC_MIN = 3 };
+enum { ORC_I8 = 0, ORC_U8 = 1, ORC_I32 = 2, ORC_U32 = 3, ORC_I64 = 4, ORC_U64 = 5, ORC_F16 = 6, ORC_F32 = 7,
+       ORC_F64 = 8, ORC_BF16 = 9 };
+/* ORC_AVG is ncclAvg: a sum divided by the group size afterwards (integer types) or with every input multiplied
+ * by 1 / size first (float types).  ORC_PREMULSUM is the device op behind ncclRedOpCreatePreMulSum: a sum of
+ * inputs multiplied by a caller's scalar (the `_x` functions take its bits). */
+enum { ORC_SUM = 0, ORC_PROD = 1, ORC_MAX = 2, ORC_MIN = 3, ORC_AVG = 4, ORC_PREMULSUM = 5 };
 
 /* Chunk geometry of a ring collective. chunk_elems is the nominal chunk
  * (stepSize*CHUNKSTEPS/sizeof(T) in the reference), align_elems the rounding
@@ -72,6 +78,12 @@ void orc_apply(int dtype, int op, const void* a, const void* b, void* out);
 /* dst[i] = op(...op(op(src0[i], src1[i]), src2[i])..., src{k-1}[i]), rounded to
  * the storage type after every op. k >= 1 (k == 1 is a copy). */
 int orc_reduce_copy(int dtype, int op, int k, const void* const* srcs, void* dst, size_t n);
+/* ... with a scalar for ORC_PREMULSUM (the bits of one element, in the low bytes).  For ORC_AVG the group is
+ * the k sources. */
+int orc_reduce_copy_x(int dtype, int op, uint64_t scalar, int k, const void* const* srcs, void* dst, size_t n);
+/* The scalar ncclAvg turns into for a group of n: n itself for integer types, 1/n rounded to the element type
+ * for float types (bits in the low bytes). */
+uint64_t orc_avg_scalar(int dtype, int n);
 /* Same result, element range split statically over nthreads host threads. */
 int orc_reduce_copy_mt(int dtype, int op, int k, const void* const* srcs, void* dst, size_t n, int nthreads);
 
@@ -88,6 +100,14 @@ int orc_all_gather(int dtype, const orc_geom* g, int64_t sendcount, const void* 
 int orc_reduce(int dtype, int op, const orc_geom* g, int64_t count, int root, const void* const* send,
                void* const* recv);
 int orc_broadcast(int dtype, const orc_geom* g, int64_t count, int root, const void* const* send, void* const* recv);
+
+/* The reducing collectives with a scalar for ORC_PREMULSUM. */
+int orc_all_reduce_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t count, const void* const* send,
+                     void* const* recv);
+int orc_reduce_scatter_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t recvcount,
+                         const void* const* send, void* const* recv);
+int orc_reduce_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t count, int root,
+                 const void* const* send, void* const* recv);
 
 /* Ring position that owns element i of an all-reduce (does the last reduction
  * and so fixes the accumulation order). Closed form, independent of the

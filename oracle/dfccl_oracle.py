@@ -13,12 +13,15 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libdfccl_oracle.so")
 
-I8, I32, F16, F32, BF16 = 0, 2, 6, 7, 9
-SUM, PROD, MAX, MIN = 0, 1, 2, 3
-DTYPES = (I8, I32, F16, F32, BF16)
+I8, U8, I32, U32, I64, U64, F16, F32, F64, BF16 = range(10)
+SUM, PROD, MAX, MIN, AVG, PREMULSUM = 0, 1, 2, 3, 4, 5
+DTYPES = (I8, I32, F16, F32, BF16)          # the five types of the headline configurations
+ALL_DTYPES = tuple(range(10))               # every ncclDataType_t
 OPS = (SUM, PROD, MAX, MIN)
-TYPE_SIZE = {I8: 1, I32: 4, F16: 2, F32: 4, BF16: 2}
-NP_STORAGE = {I8: np.int8, I32: np.int32, F16: np.uint16, F32: np.float32, BF16: np.uint16}
+FLOAT_DTYPES = (F16, F32, F64, BF16)
+TYPE_SIZE = {I8: 1, U8: 1, I32: 4, U32: 4, I64: 8, U64: 8, F16: 2, F32: 4, F64: 8, BF16: 2}
+NP_STORAGE = {I8: np.int8, U8: np.uint8, I32: np.int32, U32: np.uint32, I64: np.int64, U64: np.uint64,
+              F16: np.uint16, F32: np.float32, F64: np.float64, BF16: np.uint16}
 
 
 def build(force=False):
@@ -54,6 +57,10 @@ def lib():
         L.orc_reduce_copy.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vpp, vp, ctypes.c_size_t]
         L.orc_reduce_copy_mt.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vpp, vp, ctypes.c_size_t,
                                          ctypes.c_int]
+        u64 = ctypes.c_uint64
+        L.orc_reduce_copy_x.argtypes = [ctypes.c_int, ctypes.c_int, u64, ctypes.c_int, vpp, vp, ctypes.c_size_t]
+        L.orc_avg_scalar.argtypes = [ctypes.c_int, ctypes.c_int]
+        L.orc_avg_scalar.restype = u64
         L.orc_real_chunk.argtypes = [ctypes.c_int64] * 4
         L.orc_real_chunk.restype = ctypes.c_int64
         gp = ctypes.POINTER(Geom)
@@ -62,6 +69,9 @@ def lib():
         L.orc_all_gather.argtypes = [ctypes.c_int, gp, ctypes.c_int64, vpp, vpp]
         L.orc_reduce.argtypes = [ctypes.c_int, ctypes.c_int, gp, ctypes.c_int64, ctypes.c_int, vpp, vpp]
         L.orc_broadcast.argtypes = [ctypes.c_int, gp, ctypes.c_int64, ctypes.c_int, vpp, vpp]
+        L.orc_all_reduce_x.argtypes = [ctypes.c_int, ctypes.c_int, u64, gp, ctypes.c_int64, vpp, vpp]
+        L.orc_reduce_scatter_x.argtypes = [ctypes.c_int, ctypes.c_int, u64, gp, ctypes.c_int64, vpp, vpp]
+        L.orc_reduce_x.argtypes = [ctypes.c_int, ctypes.c_int, u64, gp, ctypes.c_int64, ctypes.c_int, vpp, vpp]
         L.orc_all_reduce_owner.argtypes = [gp, ctypes.c_int64, ctypes.c_int64]
         L.orc_cqe_encode.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.c_uint]
         L.orc_cqe_encode.restype = ctypes.c_uint64
@@ -85,29 +95,48 @@ def _check(dtype, arrays):
         assert a.dtype == NP_STORAGE[dtype], (a.dtype, dtype)
 
 
-def reduce_copy(dtype, op, srcs, nthreads=1):
-    """Fold srcs left to right with op; returns the destination array."""
+def reduce_copy(dtype, op, srcs, nthreads=1, scalar=0):
+    """Fold srcs left to right with op; returns the destination array.  op may be AVG (over the len(srcs)
+    sources) or PREMULSUM with `scalar` = the bits of one element."""
     _check(dtype, srcs)
     dst = np.empty_like(srcs[0])
-    rc = lib().orc_reduce_copy_mt(dtype, op, len(srcs), _ptrs(srcs), dst.ctypes.data, srcs[0].size, nthreads)
+    if nthreads > 1 and scalar == 0:
+        rc = lib().orc_reduce_copy_mt(dtype, op, len(srcs), _ptrs(srcs), dst.ctypes.data, srcs[0].size, nthreads)
+    else:
+        rc = lib().orc_reduce_copy_x(dtype, op, scalar, len(srcs), _ptrs(srcs), dst.ctypes.data, srcs[0].size)
     assert rc == 0
     return dst
 
 
-def all_reduce(dtype, op, geom, sends):
+def avg_scalar(dtype, n):
+    """What ncclAvg turns into for a group of n: n (integer types) or the bits of 1/n in the element type."""
+    return lib().orc_avg_scalar(dtype, n)
+
+
+def scalar_bits(dtype, value):
+    """Bits of one element of `dtype` holding `value` (for PREMULSUM)."""
+    if dtype == F16:
+        return int(f32_to_f16_bits(np.array([value], dtype=np.float32))[0])
+    if dtype == BF16:
+        return int(f32_to_bf16_bits(np.array([value], dtype=np.float32))[0])
+    a = np.array([value]).astype(NP_STORAGE[dtype])
+    return int(np.frombuffer(a.tobytes().ljust(8, b"\0"), dtype=np.uint64)[0])
+
+
+def all_reduce(dtype, op, geom, sends, scalar=0):
     _check(dtype, sends)
     recvs = [np.zeros_like(s) for s in sends]
-    rc = lib().orc_all_reduce(dtype, op, ctypes.byref(geom), sends[0].size, _ptrs(sends), _ptrs(recvs))
+    rc = lib().orc_all_reduce_x(dtype, op, scalar, ctypes.byref(geom), sends[0].size, _ptrs(sends), _ptrs(recvs))
     assert rc == 0
     return recvs
 
 
-def reduce_scatter(dtype, op, geom, sends):
+def reduce_scatter(dtype, op, geom, sends, scalar=0):
     _check(dtype, sends)
     n = geom.n_ranks
     recvcount = sends[0].size // n
     recvs = [np.zeros(recvcount, dtype=s.dtype) for s in sends]
-    rc = lib().orc_reduce_scatter(dtype, op, ctypes.byref(geom), recvcount, _ptrs(sends), _ptrs(recvs))
+    rc = lib().orc_reduce_scatter_x(dtype, op, scalar, ctypes.byref(geom), recvcount, _ptrs(sends), _ptrs(recvs))
     assert rc == 0
     return recvs
 
@@ -121,10 +150,10 @@ def all_gather(dtype, geom, sends):
     return recvs
 
 
-def reduce(dtype, op, geom, root, sends):
+def reduce(dtype, op, geom, root, sends, scalar=0):
     _check(dtype, sends)
     recvs = [np.zeros_like(s) for s in sends]
-    rc = lib().orc_reduce(dtype, op, ctypes.byref(geom), sends[0].size, root, _ptrs(sends), _ptrs(recvs))
+    rc = lib().orc_reduce_x(dtype, op, scalar, ctypes.byref(geom), sends[0].size, root, _ptrs(sends), _ptrs(recvs))
     assert rc == 0
     return recvs
 

@@ -48,6 +48,26 @@ def make(dtype, seed, n, kind="normal", sigma=1.0, small_ints=False):
     if dtype == orc.I32:
         lo, hi = (-3, 3) if small_ints else (-(1 << 20), 1 << 20)
         return integers(seed, n, lo, hi).astype(np.int32)
+    if dtype == orc.U8:
+        lo, hi = (0, 6) if small_ints else (0, 255)
+        return integers(seed, n, lo, hi).astype(np.uint8)
+    if dtype == orc.U32:
+        if small_ints:
+            return integers(seed, n, 0, 6).astype(np.uint32)
+        return (splitmix64(seed, n) & np.uint64(0xFFFFFFFF)).astype(np.uint32)  # the whole range: sums wrap
+    if dtype == orc.I64:
+        if small_ints:
+            return integers(seed, n, -3, 3)
+        return splitmix64(seed, n).view(np.int64)
+    if dtype == orc.U64:
+        if small_ints:
+            return integers(seed, n, 0, 6).astype(np.uint64)
+        return splitmix64(seed, n)
+    if dtype == orc.F64:
+        # float64 with a full mantissa, normal(0, sigma)
+        u1 = ((splitmix64(seed, n) >> np.uint64(11)).astype(np.float64) + 1.0) / float(1 << 53)
+        u2 = (splitmix64(seed ^ 0x5DEECE66D, n) >> np.uint64(11)).astype(np.float64) / float(1 << 53)
+        return sigma * np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
     x = uniform(seed, n) if kind == "uniform" else normal(seed, n, sigma)
     if dtype == orc.F32:
         return x
