@@ -25,9 +25,20 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "oracle"))
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the headline kernel from the rocprofv3 --pmc runs recorded in
-# profiles/reduce_copy_f32_sum_k2_256MiB.md (FETCH_SIZE x 1.99974 + WRITE_SIZE x 1.00000, in KiB)
-TRAFFIC_BYTES_PER_LAUNCH = int(round((262164.1 * 1.99974 + 262144.0 * 1.00000) * 1024))
+PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "reduce_copy_f32_sum_k2_256MiB.md")
+
+
+def measured_traffic_bytes():
+    """HBM bytes per launch of the headline kernel as the rocprofv3 --pmc runs measured them (FETCH_SIZE and
+    WRITE_SIZE, each scaled by what the counter reads for a plain copy of known size): the figure the profile
+    summary records on its `traffic_bytes_per_launch:` line.  None if the summary is not there."""
+    import re
+    try:
+        with open(PROFILE_SUMMARY) as f:
+            m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", f.read(), re.M)
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def bench_reduce_copy(steps, warmup, nbytes=256 << 20, k=2):
@@ -134,6 +145,20 @@ def bench_daemon_all_reduce():
     return res
 
 
+def daemon_roofline(ar):
+    """The daemon's data movement against the HBM roofline, per protocol: algorithmic bytes of the schedule
+    (direct: every input read once and every output written once, 2 * n * N * s; FIFO ring: (6n - 4) / n * N * s
+    per rank), the best time from submission on all ranks to the last callback, and the fraction of the 8 TB/s
+    peak that makes."""
+    n, nbytes = 8, 64 << 20
+    out = {"bound": "hbm", "peak": HBM_PEAK_GBPS, "unit": "GB/s", "kernel": "dfcclDaemonKernel"}
+    for label, alg in (("direct", 2 * n * nbytes), ("fifo_512KiB_chunks", (6 * n - 4) * nbytes)):
+        ms = ar[label]["ms"]
+        gbps = alg / (ms * 1e-3) / 1e9
+        out[label] = {"bytes": alg, "ms": ms, "achieved": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+    return out
+
+
 def bench_latency():
     """SQE->CQE interval of 4 KiB fp16 all-reduces over 4 virtual ranks (taken inside the library: entry
     written -> completion seen by the poller), all ranks submitting together."""
@@ -220,13 +245,14 @@ def main():
                    "bytes_counted": "(k+1)*N*sizeof(T)", "correct": rc["correct"]},
         "frac_of_hbm_peak": round(gbps_wall / HBM_PEAK_GBPS, 4),
         "roofline": {"bound": "hbm", "achieved": round(gbps_kernel, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4), "traffic": measured_traffic_bytes(),
                      "kernel": "reduceCopyKernel<f32,Sum,2>", "kernel_ms_avg": round(rc["kernel_ms_avg"], 5),
                      "kernel_ms_min": round(rc["kernel_ms_min"], 5),
                      "kernel_ms_avg_each_launch_bracketed_by_events": round(rc["kernel_ms_avg_bracketed"], 5)},
     }
     if not args.skip_daemon:
         line["daemon_all_reduce"] = bench_daemon_all_reduce()
+        line["daemon_roofline"] = daemon_roofline(line["daemon_all_reduce"])
         line["sqe_to_cqe_latency"] = bench_latency()
         line["disordered_small_collectives"] = bench_disordered()
         line["gradient_buckets"] = bench_buckets()

@@ -6,5 +6,6 @@ and the benchmark; torch is only used for device memory and streams.
 """
 from .api import (  # noqa: F401
     DTYPE_OF, NcclError, RankCtx, UniqueId, VirtualComm, check, nccl_dtype, reduce_copy,
-    ncclSum, ncclProd, ncclMax, ncclMin, ncclInt8, ncclInt32, ncclFloat16, ncclFloat32, ncclBfloat16,
+    ncclSum, ncclProd, ncclMax, ncclMin, ncclAvg, ncclInt8, ncclUint8, ncclInt32, ncclUint32, ncclInt64, ncclUint64,
+    ncclFloat16, ncclFloat32, ncclFloat64, ncclBfloat16,
 )

@@ -38,6 +38,8 @@ SIGNATURES = {
     "ncclCommCount": (_int, [_vp, ctypes.POINTER(_int)]),
     "ncclCommUserRank": (_int, [_vp, ctypes.POINTER(_int)]),
     "ncclGetErrorString": (ctypes.c_char_p, [_int]),
+    "ncclRedOpCreatePreMulSum": (_int, [ctypes.POINTER(_int), _vp, _int, _int, _vp]),
+    "ncclRedOpDestroy": (_int, [_int, _vp]),
     "ofcclInitRankCtx": (_int, [ctypes.POINTER(_vp), _int]),
     "ofcclFinalizeRankCtx7StartHostThrds": (_int, [_vp]),
     "ofcclPrepareDone": (_int, [_vp]),

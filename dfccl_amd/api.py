@@ -9,11 +9,17 @@ import torch
 from . import _lib
 from ._lib import CALLBACK, CollGeometry, Stats, UniqueId
 
-ncclSum, ncclProd, ncclMax, ncclMin = 0, 1, 2, 3
-ncclInt8, ncclInt32, ncclFloat16, ncclFloat32, ncclBfloat16 = 0, 2, 6, 7, 9
+ncclSum, ncclProd, ncclMax, ncclMin, ncclAvg = 0, 1, 2, 3, 4
+(ncclInt8, ncclUint8, ncclInt32, ncclUint32, ncclInt64, ncclUint64, ncclFloat16, ncclFloat32, ncclFloat64,
+ ncclBfloat16) = range(10)
+ncclScalarDevice, ncclScalarHostImmediate = 0, 1
 
-DTYPE_OF = {torch.int8: ncclInt8, torch.int32: ncclInt32, torch.float16: ncclFloat16,
-            torch.float32: ncclFloat32, torch.bfloat16: ncclBfloat16}
+DTYPE_OF = {torch.int8: ncclInt8, torch.uint8: ncclUint8, torch.int32: ncclInt32, torch.int64: ncclInt64,
+            torch.float16: ncclFloat16, torch.float32: ncclFloat32, torch.float64: ncclFloat64,
+            torch.bfloat16: ncclBfloat16}
+for _name, _code in (("uint32", ncclUint32), ("uint64", ncclUint64)):  # (newer torch versions have these)
+    if hasattr(torch, _name):
+        DTYPE_OF[getattr(torch, _name)] = _code
 
 
 class NcclError(RuntimeError):
@@ -45,9 +51,10 @@ def _dev_ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
-def reduce_copy(srcs, dst, op=ncclSum, chunk_bytes=0, stream=None):
+def reduce_copy(srcs, dst, op=ncclSum, chunk_bytes=0, stream=None, dtype=None):
     """dst = srcs[0] (op) srcs[1] (op) ... folded left to right (dfcclReduceCopy). Asynchronous on `stream`
-    (default: torch's current stream)."""
+    (default: torch's current stream).  `dtype` overrides the ncclDataType_t taken from the tensors (for element
+    types torch has no tensor type for, held in tensors of the same width)."""
     lib = _lib.load()
     n = dst.numel()
     for s in srcs:
@@ -56,8 +63,8 @@ def reduce_copy(srcs, dst, op=ncclSum, chunk_bytes=0, stream=None):
     arr = (ctypes.c_void_p * len(srcs))(*[s.data_ptr() for s in srcs])
     if stream is None:
         stream = torch.cuda.current_stream(dst.device)
-    check(lib.dfcclReduceCopy(arr, len(srcs), _dev_ptr(dst), n, nccl_dtype(dst), op, chunk_bytes,
-                              ctypes.c_void_p(stream.cuda_stream)), "dfcclReduceCopy")
+    check(lib.dfcclReduceCopy(arr, len(srcs), _dev_ptr(dst), n, nccl_dtype(dst) if dtype is None else dtype, op,
+                              chunk_bytes, ctypes.c_void_p(stream.cuda_stream)), "dfcclReduceCopy")
 
 
 class VirtualComm:
@@ -79,6 +86,17 @@ class VirtualComm:
         """The nranks handles of one fresh communicator, index = rank."""
         uid = cls.unique_id()
         return [cls(nranks, uid, r) for r in range(nranks)]
+
+    def create_premul_sum(self, dtype, scalar_bytes):
+        """ncclRedOpCreatePreMulSum with the scalar given as the bytes of one element; returns the op value."""
+        op = ctypes.c_int()
+        buf = ctypes.create_string_buffer(bytes(scalar_bytes).ljust(8, b"\0"), 8)
+        check(_lib.load().ncclRedOpCreatePreMulSum(ctypes.byref(op), ctypes.cast(buf, ctypes.c_void_p), dtype,
+                                                   ncclScalarHostImmediate, self.handle), "ncclRedOpCreatePreMulSum")
+        return op.value
+
+    def destroy_op(self, op):
+        check(_lib.load().ncclRedOpDestroy(op, self.handle), "ncclRedOpDestroy")
 
     def destroy(self):
         if self.handle:

@@ -54,7 +54,8 @@ struct SweepGeom {
   uint64_t ctr;                      // the rank's tile counter
   int n, C, ch, es;                  // n: sources folded (1 = plain copy)
   int me, dtype, op, nd;             // nd: destinations written
-  int tn, tme, pad0, pad1;           // a loop holds C * tn chunks, mine is number tme of every channel slot
+  int tn, tme, scaleKind, pad1;      // a loop holds C * tn chunks, mine is number tme of every channel slot
+  uint64_t scaleBits;                // scaled sums: see Scale in reduce_ops.h
   uint64_t src[kMaxDirectRanks];     // the send buffers in fold order: in[me + 1], in[me + 2], ..., in[me]
   uint64_t dst[kMaxDirectRanks];     // every rank's receive buffer
 };
@@ -595,6 +596,21 @@ __device__ __forceinline__ void copySlice(const void* s0, void* d0, void* d1, si
   }
 }
 
+// Expands CALL once for every element type of ncclDataType_t, with DT the type's number as a constant.
+#define DFCCL_FOR_DTYPE(dtype, CALL)                        \
+  switch (dtype) {                                          \
+    case kF32: { constexpr int DT = kF32; CALL; } break;    \
+    case kBF16: { constexpr int DT = kBF16; CALL; } break;  \
+    case kF16: { constexpr int DT = kF16; CALL; } break;    \
+    case kI32: { constexpr int DT = kI32; CALL; } break;    \
+    case kI8: { constexpr int DT = kI8; CALL; } break;      \
+    case kU8: { constexpr int DT = kU8; CALL; } break;      \
+    case kU32: { constexpr int DT = kU32; CALL; } break;    \
+    case kI64: { constexpr int DT = kI64; CALL; } break;    \
+    case kU64: { constexpr int DT = kU64; CALL; } break;    \
+    default: { constexpr int DT = kF64; CALL; } break;      \
+  }
+
 // One slice: 1 or 2 sources into 1 or 2 destinations (s1 / d1 may be null).
 __device__ __forceinline__ void moveSlice(int dtype, int op, const void* s0, const void* s1, void* d0, void* d1,
                                           size_t nbytes, int tid) {
@@ -602,13 +618,37 @@ __device__ __forceinline__ void moveSlice(int dtype, int op, const void* s0, con
     copySlice(s0, d0, d1, nbytes, tid);
     return;
   }
-  switch (dtype) {
-    case kF32: moveReduceOp<kF32>(op, s0, s1, d0, d1, nbytes, tid); break;
-    case kBF16: moveReduceOp<kBF16>(op, s0, s1, d0, d1, nbytes, tid); break;
-    case kF16: moveReduceOp<kF16>(op, s0, s1, d0, d1, nbytes, tid); break;
-    case kI32: moveReduceOp<kI32>(op, s0, s1, d0, d1, nbytes, tid); break;
-    default: moveReduceOp<kI8>(op, s0, s1, d0, d1, nbytes, tid); break;
+  DFCCL_FOR_DTYPE(dtype, moveReduceOp<DT>(op, s0, s1, d0, d1, nbytes, tid));
+}
+
+// The same for a slice of a scaled sum (ncclAvg, PreMulSum) that reads a user input or produces the final value:
+// source 0 is the user's buffer whenever a step has one (su.preMask says whether it is multiplied).
+template <int DT>
+__device__ __forceinline__ void moveScaled(const void* s0, const void* s1, void* d0, void* d1, size_t nbytes, int tid,
+                                           const ScaleUse& su) {
+  if (s1 != nullptr) {
+    const void* s[2] = {s0, s1};
+    if (d1 != nullptr) {
+      void* d[2] = {d0, d1};
+      reduceCopyWG<DT, kSum, 2, 2, kDaemonUnroll, false, true>(s, d, nbytes, tid, kWgThreads, su);
+    } else {
+      void* d[1] = {d0};
+      reduceCopyWG<DT, kSum, 2, 1, kDaemonUnroll, false, true>(s, d, nbytes, tid, kWgThreads, su);
+    }
+  } else {
+    const void* s[1] = {s0};
+    if (d1 != nullptr) {
+      void* d[2] = {d0, d1};
+      reduceCopyWG<DT, kSum, 1, 2, kDaemonUnroll, false, true>(s, d, nbytes, tid, kWgThreads, su);
+    } else {
+      void* d[1] = {d0};
+      reduceCopyWG<DT, kSum, 1, 1, kDaemonUnroll, false, true>(s, d, nbytes, tid, kWgThreads, su);
+    }
   }
+}
+__device__ __forceinline__ void moveSliceScaled(int dtype, const void* s0, const void* s1, void* d0, void* d1,
+                                                size_t nbytes, int tid, const ScaleUse& su) {
+  DFCCL_FOR_DTYPE(dtype, moveScaled<DT>(s0, s1, d0, d1, nbytes, tid, su));
 }
 
 // Direct protocol data movement.  A "tile" is one rank's chunk of one loop.
@@ -625,10 +665,17 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
 // re-read src[0] (they hit in cache) so that every array element is defined: predicated loads made the compiler
 // keep the packs in scratch.  A destination may be one of the sources (in place): each thread reads a pack
 // before it writes it, and no other thread touches that pack.
-template <int DT, int OP, int NS>
+// SC: a scaled sum (OP is kSum): every source is a user input and is multiplied by the scalar first (kScalePre), or
+// the result is divided by the group size (kScalePost, integer types).
+template <int DT, int OP, int NS, bool SC = false>
 __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks], const uint64_t (&dst)[kMaxDirectRanks],
-                                         int n, int nd, int64_t byteOff, size_t nbytes, int tid, int nthr) {
+                                         int n, int nd, int64_t byteOff, size_t nbytes, int tid, int nthr,
+                                         int scaleKind = kScaleNone, uint64_t scaleBits = 0) {
   constexpr int ES = typeSize(DT);
+  const bool pre = SC && scaleKind == kScalePre;
+  const bool post = SC && !isFloatType(DT) && scaleKind == kScalePost;
+  const u32x4 factor = splatScalar<DT>(scaleBits);
+  const int divisor = (int)scaleBits;
   uint64_t align = (uint64_t)byteOff;
 #pragma unroll
   for (int j = 0; j < NS; j++) align |= (j < n ? src[j] : 0);
@@ -642,10 +689,15 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
       u32x4 v[NS];
 #pragma unroll
       for (int j = 0; j < NS; j++) v[j] = loadPack<true>((const char*)(j < n ? src[j] : src[0]) + byteOff, i);
+      if (pre) {
+#pragma unroll
+        for (int j = 0; j < NS; j++) v[j] = packOp<DT, kProd>(v[j], factor);
+      }
       u32x4 acc = v[0];
 #pragma unroll
       for (int j = 1; j < NS; j++)
         if (j < n) acc = packOp<DT, OP>(acc, v[j]);
+      if (post) acc = packPostDiv<DT>(acc, divisor);
 #pragma unroll
       for (int j = 0; j < kMaxDirectRanks; j++)
         if (j < nd) storePack<false>((char*)dst[j] + byteOff, i, acc);
@@ -655,10 +707,16 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
   const size_t first = doneBytes / ES, nelem = nbytes / ES;
 #pragma clang loop vectorize(disable) interleave(disable) unroll(disable)
   for (size_t i = first + tid; i < nelem; i += nthr) {
-    uint32_t acc = loadElem<ES>((const char*)src[0] + byteOff, i);
+    uint64_t acc = loadElem<ES>((const char*)src[0] + byteOff, i);
+    if (pre) acc = elemPreMul<DT>(acc, scaleBits);
 #pragma unroll
     for (int j = 1; j < NS; j++)
-      if (j < n) acc = wordOp<DT, OP>(acc, loadElem<ES>((const char*)src[j] + byteOff, i));
+      if (j < n) {
+        uint64_t v = loadElem<ES>((const char*)src[j] + byteOff, i);
+        if (pre) v = elemPreMul<DT>(v, scaleBits);
+        acc = elemOp<DT, OP>(acc, v);
+      }
+    if (post) acc = elemPostDiv<DT>(acc, divisor);
 #pragma unroll
     for (int j = 0; j < kMaxDirectRanks; j++)
       if (j < nd) storeElem<ES>((char*)dst[j] + byteOff, i, acc);
@@ -677,7 +735,7 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
 //    decides when the collective is done.  The next tile is requested while the current one is folded.  Every
 //    workgroup draws exactly one number past the end per instance, so the counter advances by exactly T.
 // At most maxTiles tiles are processed; `finished` says that no tile is left.
-template <int DT, int OP, int NS>
+template <int DT, int OP, int NS, bool SC = false>
 __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, int64_t& posInOut, int64_t maxTiles,
                                            int tid, int nthr, int64_t& tilesDone, bool& finished) {
   const bool dynamic = g.C > 1;
@@ -714,7 +772,9 @@ __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, 
     const int64_t real = ((int64_t)l == g.L - 1) ? g.lastReal : g.chunkElems;
     const int64_t off = (int64_t)l * g.loop + ((int64_t)slot * g.tn + g.tme) * real;
     const int64_t nelem = (g.count - off < real) ? g.count - off : real;
-    if (nelem > 0) foldTile<DT, OP, NS>(g.src, g.dst, g.n, g.nd, off * g.es, (size_t)(nelem * g.es), tid, nthr);
+    if (nelem > 0)
+      foldTile<DT, OP, NS, SC>(g.src, g.dst, g.n, g.nd, off * g.es, (size_t)(nelem * g.es), tid, nthr, g.scaleKind,
+                               g.scaleBits);
     done++;
     if (prefetch) {
       if (tid == 0) slots[par] = nxt;
@@ -729,12 +789,12 @@ __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, 
   finished = fin;
 }
 
-template <int DT, int OP>
+template <int DT, int OP, bool SC = false>
 __device__ __forceinline__ void sweepFold(const SweepGeom& g, uint64_t* slots, int64_t& pos, int64_t maxTiles, int tid,
                                           int nthr, int64_t& tilesDone, bool& finished) {
-  if (g.n <= 2) sweepFoldN<DT, OP, 2>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
-  else if (g.n <= 4) sweepFoldN<DT, OP, 4>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
-  else sweepFoldN<DT, OP, 8>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
+  if (g.n <= 2) sweepFoldN<DT, OP, 2, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
+  else if (g.n <= 4) sweepFoldN<DT, OP, 4, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
+  else sweepFoldN<DT, OP, 8, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
 }
 
 template <int DT>
@@ -756,13 +816,11 @@ __device__ __forceinline__ void sweepFoldAny(const SweepGeom& g, uint64_t* slots
     sweepFoldN<kI8, kSum, 1>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
     return;
   }
-  switch (g.dtype) {
-    case kF32: sweepFoldOp<kF32>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
-    case kBF16: sweepFoldOp<kBF16>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
-    case kF16: sweepFoldOp<kF16>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
-    case kI32: sweepFoldOp<kI32>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
-    default: sweepFoldOp<kI8>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
+  if (g.scaleKind != kScaleNone) {  // ncclAvg / PreMulSum: a sum with a scale
+    DFCCL_FOR_DTYPE(g.dtype, (sweepFold<DT, kSum, true>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished)));
+    return;
   }
+  DFCCL_FOR_DTYPE(g.dtype, sweepFoldOp<DT>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished));
 }
 
 // ------------------------------------------------------------- FIFO ring protocol
@@ -831,7 +889,22 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
         else s0 = fifoIn;
         if (d.useOut) { d0 = recvbuff + (d.outOff + off) * es; d1 = fifoOut; }
         else d0 = fifoOut;
-        if (s0 != nullptr && d0 != nullptr) moveSlice(P.dtype, P.op, s0, s1, d0, d1, (size_t)(len * es), tid);
+        if (s0 != nullptr && d0 != nullptr) {
+          // a scaled sum (ncclAvg / PreMulSum) multiplies the user's input where it enters (source 0 of a step that
+          // reads it) and divides where the final value is produced
+          const bool scaledStep = P.scaleKind != kScaleNone && n > 1 &&
+                                  ((P.scaleKind == kScalePre && d.useIn) || (P.scaleKind == kScalePost && d.post));
+          if (scaledStep) {
+            ScaleUse su;
+            su.scale.kind = P.scaleKind;
+            su.scale.bits = P.scaleBits;
+            su.preMask = d.useIn ? 1u : 0u;
+            su.post = d.post != 0;
+            moveSliceScaled(P.dtype, s0, s1, d0, d1, (size_t)(len * es), tid, su);
+          } else {
+            moveSlice(P.dtype, P.op, s0, s1, d0, d1, (size_t)(len * es), tid);
+          }
+        }
         if (d.recv || d.send) {
           __syncthreads();  // every thread's loads and stores of this slice are done
           if (tid == 0) {
@@ -908,7 +981,9 @@ __device__ __forceinline__ void layOutSweep(SweepGeom& g, const CollPlan& P, int
   g.me = me;
   g.dtype = P.dtype;
   g.op = P.op;
-  g.pad0 = g.pad1 = 0;
+  g.scaleKind = (folds && n > 1) ? P.scaleKind : (int)kScaleNone;
+  g.scaleBits = P.scaleBits;
+  g.pad1 = 0;
 }
 
 // Collectives in which the virtual ranks, whose buffers share one HBM, read each

@@ -118,7 +118,9 @@ struct alignas(16) CollPlan {
   ConnFlags* recvFlags;
   uint64_t* doneCounter;   // workgroups that finished an instance, monotonic
   // direct protocol (peers read each other's buffers, no FIFO)
-  int32_t proto, pad2;
+  int32_t proto;
+  int32_t scaleKind;       // a Sum with a scale (ncclAvg, PreMulSum): kScaleNone / kScalePre / kScalePost of reduce_ops.h
+  uint64_t scaleBits;      // its scalar: one element of dtype in the low bytes, or the divisor
   PeerPub* pubs;           // [nRanks][nChannels]
   uint64_t* p1;            // [nRanks][nChannels] loops whose own chunk is folded and stored everywhere
   int64_t loopsPerInstance;

@@ -64,6 +64,7 @@ struct StepDesc {
   int send;      // put the result into the FIFO towards the next rank
   int useIn;     // read the user's send buffer at inOff
   int useOut;    // write the user's receive buffer at outOff
+  int post;      // this step produces the final value of a reduction (the reference's postOp = true)
   int64_t inOff;
   int64_t outOff;
   int64_t nelem; // may be <= 0: nothing to do for this rank/step (both ends agree)
@@ -74,7 +75,7 @@ struct StepDesc {
 DFCCL_HD StepDesc describeStep(int kind, int n, int rank, int root, int nChannels, int bid, int64_t count,
                                int64_t gridOffset, int64_t real, int step, int inPlace) {
   StepDesc d;
-  d.recv = d.send = d.useIn = d.useOut = 0;
+  d.recv = d.send = d.useIn = d.useOut = d.post = 0;
   d.inOff = d.outOff = 0;
   d.nelem = 0;
   (void)nChannels;
@@ -90,7 +91,7 @@ DFCCL_HD StepDesc describeStep(int kind, int n, int rank, int root, int nChannel
     int chunk;
     if (step == 0) { chunk = (rank + n - 1) % n; d.useIn = 1; d.send = 1; }
     else if (step <= n - 2) { chunk = (rank + n - (step + 1)) % n; d.recv = 1; d.useIn = 1; d.send = 1; }
-    else if (step == n - 1) { chunk = rank; d.recv = 1; d.useIn = 1; d.useOut = 1; d.send = 1; }
+    else if (step == n - 1) { chunk = rank; d.recv = 1; d.useIn = 1; d.useOut = 1; d.send = 1; d.post = 1; }
     else if (step <= 2 * n - 3) { chunk = (rank + n - (step - n + 1)) % n; d.recv = 1; d.useOut = 1; d.send = 1; }
     else { chunk = (rank + 1) % n; d.recv = 1; d.useOut = 1; }
     const int64_t off = gridOffset + (int64_t)bid * n * real + (int64_t)chunk * real;
@@ -104,7 +105,7 @@ DFCCL_HD StepDesc describeStep(int kind, int n, int rank, int root, int nChannel
     int dest;
     if (step == 0) { dest = (rank + n - 1) % n; d.useIn = 1; d.send = 1; }
     else if (step <= n - 2) { dest = (rank + n - (step + 1)) % n; d.recv = 1; d.useIn = 1; d.send = 1; }
-    else { dest = rank; d.recv = 1; d.useIn = 1; d.useOut = 1; }
+    else { dest = rank; d.recv = 1; d.useIn = 1; d.useOut = 1; d.post = 1; }
     d.inOff = chunkOff + (int64_t)dest * count;
     d.outOff = chunkOff;
   } else if (kind == kAllGather) {
@@ -117,7 +118,7 @@ DFCCL_HD StepDesc describeStep(int kind, int n, int rank, int root, int nChannel
   } else if (kind == kReduce) {
     d.inOff = d.outOff = chunkOff;
     if ((rank + n - 1) % n == root) { d.useIn = 1; d.send = 1; }
-    else if (rank == root) { d.recv = 1; d.useIn = 1; d.useOut = 1; }
+    else if (rank == root) { d.recv = 1; d.useIn = 1; d.useOut = 1; d.post = 1; }
     else { d.recv = 1; d.useIn = 1; d.send = 1; }
   } else {  // broadcast
     d.inOff = d.outOff = chunkOff;

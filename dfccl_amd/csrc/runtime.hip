@@ -27,6 +27,7 @@
 #include <vector>
 
 #include "../../include/ofccl.h"
+#include "avg_scale.h"
 #include "dfccl_common.h"
 
 #define DFCCL_API extern "C" __attribute__((visibility("default")))
@@ -69,11 +70,6 @@ static int typeSizeOf(int dt) {
   }
 }
 
-// dtypes the reduce kernels implement; copies (all-gather, broadcast) take any type
-static bool reduceDtypeSupported(int dt) {
-  return dt == ncclInt8 || dt == ncclInt32 || dt == ncclFloat16 || dt == ncclFloat32 || dt == ncclBfloat16;
-}
-
 // ------------------------------------------------------------------ communicators
 
 struct CommGroup {
@@ -87,7 +83,9 @@ struct CommGroup {
   // a rank context that ran this collective has been destroyed: the counters in the group's device memory no
   // longer match a fresh context's, so the communicator cannot be registered again
   bool retired = false;
-  int kind = 0, dtypeUser = 0, op = 0, root = 0;
+  int kind = 0, dtypeUser = 0, op = 0, root = 0;  // op: the element op the kernels apply (Sum for the scaled sums)
+  int scaleKind = kScaleNone;                      // ncclAvg / PreMulSum: see Scale in reduce_ops.h
+  uint64_t scaleBits = 0;
   size_t countUser = 0;
   // derived plan
   int dtype = 0, elemSize = 1, nChannels = 1, slicesPerChunk = 1, fifoSlots = 1;
@@ -109,6 +107,9 @@ struct ncclComm {
   dfccl::CommGroup* group;
   int rank;
   bool registered;
+  // reduction operators made by ncclRedOpCreatePreMulSum: op value - ncclNumOps -> {datatype, scalar bits}
+  std::map<int, std::pair<int, uint64_t>> userOps;
+  int nextUserOp = 0;
 };
 
 namespace dfccl {
@@ -555,11 +556,30 @@ static ncclResult_t prepareColl(int kind, size_t count, int dtype, int op, int r
   CommGroup* g = comm->group;
   if (root < 0 || root >= g->nRanks) return ncclInvalidArgument;
   if (dtype < 0 || dtype >= ncclNumTypes) return ncclInvalidArgument;
-  if (op < 0 || op >= ncclNumOps) return ncclInvalidArgument;
   const bool reduces = (kind == kAllReduce || kind == kReduceScatter || kind == kReduce);
-  if (reduces && (op == ncclAvg || !reduceDtypeSupported(dtype))) return ncclInvalidArgument;
+  if (op < 0) return ncclInvalidArgument;
   if (comm->registered) return ncclInvalidUsage;  // one communicator per collective
   if (comm->rank != ctx->rank) return ncclInvalidArgument;
+  // What the op becomes on the device (hostToDevRedOp, src/enqueue.cc:1305-1371): the four element ops as they
+  // are; ncclAvg a Sum that divides the result by nRanks (integer types) or multiplies every input by 1/nRanks
+  // first (float types); an operator made by ncclRedOpCreatePreMulSum a Sum of inputs times its scalar.
+  int devOp = reduces ? op : (int)ncclSum;
+  Scale scale;
+  scale.kind = kScaleNone;
+  scale.bits = 0;
+  if (reduces && op == ncclAvg) {
+    devOp = ncclSum;
+    scale = dfcclAvgScale(dtype, g->nRanks);
+  } else if (reduces && op >= ncclNumOps) {
+    auto it = comm->userOps.find(op - (int)ncclNumOps);
+    if (it == comm->userOps.end()) return ncclInvalidArgument;
+    if (it->second.first != dtype) return ncclInvalidArgument;  // made for another datatype (enqueue.cc:1361-1365)
+    devOp = ncclSum;
+    scale.kind = kScalePre;
+    scale.bits = it->second.second;
+  } else if (op >= ncclNumOps) {
+    return ncclInvalidArgument;
+  }
   {
     std::lock_guard<std::mutex> lk(g->mu);
     if (g->device != ctx->device) return ncclInvalidUsage;
@@ -567,14 +587,18 @@ static ncclResult_t prepareColl(int kind, size_t count, int dtype, int op, int r
     if (!g->planned) {
       g->kind = kind;
       g->dtypeUser = dtype;
-      g->op = reduces ? op : (int)ncclSum;
+      g->op = devOp;
+      g->scaleKind = scale.kind;
+      g->scaleBits = scale.bits;
       g->root = root;
       g->countUser = count;
       planGroup(g);
       g->planned = true;
     } else if (g->kind != kind || g->dtypeUser != dtype || g->countUser != count || g->root != root ||
-               (reduces && g->op != op)) {
-      return ncclInvalidArgument;  // the ranks of a communicator must describe the same collective
+               (reduces && (g->op != devOp || g->scaleKind != scale.kind || g->scaleBits != scale.bits))) {
+      // the ranks of a communicator must describe the same collective (for a PreMulSum operator that includes
+      // the scalar: the virtual ranks fold each other's inputs, so one scalar serves the whole communicator)
+      return ncclInvalidArgument;
     }
   }
   comm->registered = true;
@@ -740,7 +764,11 @@ DFCCL_API ncclResult_t ncclCommInitRank(ncclComm_t* comm, int nranks, ncclUnique
     if (g->nRanks != nranks || g->device != device) return ncclInvalidArgument;
   }
   g->handles++;
-  *comm = new ncclComm{g, rank, false};
+  ncclComm* c = new ncclComm();
+  c->group = g;
+  c->rank = rank;
+  c->registered = false;
+  *comm = c;
   return ncclSuccess;
 }
 
@@ -787,6 +815,31 @@ DFCCL_API ncclResult_t ncclCommCount(const ncclComm_t comm, int* count) {
 DFCCL_API ncclResult_t ncclCommUserRank(const ncclComm_t comm, int* rank) {
   if (comm == nullptr || rank == nullptr) return ncclInvalidArgument;
   *rank = comm->rank;
+  return ncclSuccess;
+}
+
+// A reduction operator that multiplies every input by *scalar before summing (src/nccl.h.in:169-180,
+// src/enqueue.cc:1443-1490).  The scalar is read now (ncclScalarHostImmediate); one that lives in device memory
+// and is read while the collective runs is not supported on this path, where a collective is prepared once and
+// run many times.
+DFCCL_API ncclResult_t ncclRedOpCreatePreMulSum(ncclRedOp_t* op, void* scalar, ncclDataType_t datatype,
+                                                ncclScalarResidence_t residence, ncclComm_t comm) {
+  if (op == nullptr || scalar == nullptr || comm == nullptr) return ncclInvalidArgument;
+  const int es = typeSizeOf((int)datatype);
+  if (es == 0) return ncclInvalidArgument;
+  if (residence != ncclScalarHostImmediate) return ncclInvalidArgument;
+  uint64_t bits = 0;
+  memcpy(&bits, scalar, (size_t)es);
+  const int ix = comm->nextUserOp++;
+  comm->userOps[ix] = std::make_pair((int)datatype, bits);
+  *op = (ncclRedOp_t)((int)ncclNumOps + ix);
+  return ncclSuccess;
+}
+
+DFCCL_API ncclResult_t ncclRedOpDestroy(ncclRedOp_t op, ncclComm_t comm) {
+  if (comm == nullptr) return ncclInvalidArgument;
+  if ((int)op < (int)ncclNumOps) return ncclInvalidArgument;  // built-in operators cannot be destroyed
+  if (comm->userOps.erase((int)op - (int)ncclNumOps) == 0) return ncclInvalidArgument;
   return ncclSuccess;
 }
 
@@ -883,7 +936,7 @@ DFCCL_API ncclResult_t ofcclFinalizeRankCtx7StartHostThrds(ofcclRankCtx_t c) {
     p.slotBytes = g->slotBytes; p.fifoChanStride = g->chanStride;
     p.sendFifo = g->fifo ? g->fifo + (size_t)rank * g->nChannels * g->chanStride : nullptr;
     p.recvFifo = g->fifo ? g->fifo + (size_t)prev * g->nChannels * g->chanStride : nullptr;
-    p.proto = g->proto; p.pad2 = 0; p.pubs = g->pubs; p.p1 = g->p1;
+    p.proto = g->proto; p.scaleKind = g->scaleKind; p.scaleBits = g->scaleBits; p.pubs = g->pubs; p.p1 = g->p1;
     p.loopsPerInstance = g->loopsPerInstance;
     p.lastChunkElems = g->lastChunkElems;
     p.tileCtr = g->tileCtrs ? g->tileCtrs + (size_t)rank * 16 : nullptr;

@@ -23,9 +23,13 @@ class VirtualRing:
         self.finalized = False
 
     # -- registration -----------------------------------------------------------
-    def prepare(self, coll_id, kind, count, dtype, op=api.ncclSum, root=0):
+    def prepare(self, coll_id, kind, count, dtype, op=api.ncclSum, root=0, premul=None):
+        """premul: the bytes of one element; every rank then makes a PreMulSum operator with that scalar on its
+        communicator handle and registers the collective with it (op is ignored)."""
         comms = api.VirtualComm.create_all(self.n)
         for r, ctx in enumerate(self.ctxs):
+            if premul is not None:
+                op = comms[r].create_premul_sum(dtype, premul)
             if kind == "all_reduce":
                 ctx.prepare_all_reduce(count, dtype, op, comms[r], coll_id)
             elif kind == "reduce_scatter":

@@ -48,8 +48,9 @@ typedef enum { /* nccl.h.in:113-128 */
   ncclProd = 1,
   ncclMax = 2,
   ncclMin = 3,
-  ncclAvg = 4, /* not on this path: Prepare returns ncclInvalidArgument */
-  ncclNumOps = 5
+  ncclAvg = 4,
+  ncclNumOps = 5, /* operators made by ncclRedOpCreatePreMulSum have values from here on */
+  ncclMaxRedOp = 0x7fffffff
 } ncclRedOp_t;
 
 typedef enum { /* nccl.h.in:131-146 */
@@ -82,6 +83,25 @@ ncclResult_t ncclCommCount(const ncclComm_t comm, int* count);                  
 ncclResult_t ncclCommUserRank(const ncclComm_t comm, int* rank);                           /* nccl.h.in:108 */
 const char* ncclGetErrorString(ncclResult_t result);                                       /* nccl.h.in:92 */
 
+/* ---- reduction operators with a scalar (nccl.h.in:148-180) ----------------
+ * ncclRedOpCreatePreMulSum makes an operator that multiplies every input by
+ * *scalar (one element of `datatype`) before summing, for collectives prepared
+ * on `comm` with that datatype (src/enqueue.cc:1443-1490; device semantics
+ * src/include/reduce_kernel.h:503-668: one rounded multiply in the element type).
+ * Differences on this path: the scalar is read when the operator is created
+ * (ncclScalarHostImmediate; ncclScalarDevice returns ncclInvalidArgument,
+ * because a collective is prepared once and run many times), and all ranks of
+ * a communicator must give the same scalar (the virtual ranks fold each
+ * other's inputs): Prepare returns ncclInvalidArgument otherwise.
+ * ncclAvg needs none of this: Prepare turns it into a sum that is divided by
+ * the number of ranks afterwards (integer types, C++ integer division) or
+ * whose inputs are multiplied by 1/nranks first (float types), as
+ * src/enqueue.cc:1326-1357 does. */
+typedef enum { ncclScalarDevice = 0, ncclScalarHostImmediate = 1 } ncclScalarResidence_t; /* nccl.h.in:148-156 */
+ncclResult_t ncclRedOpCreatePreMulSum(ncclRedOp_t* op, void* scalar, ncclDataType_t datatype,
+                                      ncclScalarResidence_t residence, ncclComm_t comm);   /* nccl.h.in:169 */
+ncclResult_t ncclRedOpDestroy(ncclRedOp_t op, ncclComm_t comm);                            /* nccl.h.in:179 */
+
 /* ---- rank context ---------------------------------------------------------*/
 
 /* Allocates a rank context for virtual rank `rank` on the current HIP device.
@@ -108,7 +128,8 @@ ncclResult_t ofcclDestroy(ofcclRankCtx_t rankCtx);
  * may be registered once (and not again after a rank context that ran its
  * collective has been destroyed: create a new communicator), root / dtype / op in range.  Buffers are given at
  * Run time.  Unlike the reference (which drops `op` and always sums,
- * src/enqueue_ofccl.cc:211-215) Sum / Prod / Max / Min are honoured. */
+ * src/enqueue_ofccl.cc:211-215) the op is honoured: Sum / Prod / Max / Min / Avg and operators made by
+ * ncclRedOpCreatePreMulSum, on every ncclDataType_t. */
 ncclResult_t ofcclPrepareReduce(size_t count, ncclDataType_t datatype, ncclRedOp_t op, int root, ncclComm_t comm,
                                 int collId, ofcclRankCtx_t rankCtx);                       /* nccl.h.in:253 */
 ncclResult_t ofcclPrepareBcast(size_t count, ncclDataType_t datatype, int root, ncclComm_t comm, int collId,

@@ -34,15 +34,18 @@ def _enter_emulation():
     lib.LIB_PATH = EMULATION_LIB
     os.environ.setdefault("NCCL_MAX_NCHANNELS", "2")  # every workgroup is a few hundred OS threads there
     os.environ.setdefault("DFCCL_STATS_WAIT_MS", "5000")  # and answers a request for its counters slowly
+    os.environ.setdefault("DFCCL_RC_MAX_WGS", "3")        # the one-shot reduce-copy kernel: 3 workgroups of 512 OS threads
     gpu_util.EMULATED = True
     api._dev_ptr = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())  # host memory is device memory there
     gpu_util.DEVICE = "cpu"
+
+    emul = ctypes.CDLL(EMULATION_LIB)
 
     class _NoStream:
         cuda_stream = 0
 
         def synchronize(self):
-            pass
+            emul.emulNullStreamSynchronize()  # kernels launched on the null stream run as threads of their own
 
     torch.cuda.current_stream = lambda *a, **k: _NoStream()
     torch.cuda.synchronize = lambda *a, **k: None

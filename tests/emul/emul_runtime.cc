@@ -205,6 +205,8 @@ static void startWatchdog() {
 }  // namespace emul
 
 extern "C" void emulDumpThreads() { emul::dumpThreads(stderr); }
+// for callers outside C++ (the Python tests): wait for the kernels launched on the null stream
+extern "C" void emulNullStreamSynchronize() { (void)hipStreamSynchronize(nullptr); }
 
 static size_t roundUp(size_t n, size_t a) { return (n + a - 1) / a * a; }
 

@@ -80,10 +80,118 @@ def test_all_reduce_fp32_sum_sizes_and_ranks(n, count):
     check("all_reduce", orc.F32, orc.SUM, n, count, reps=2)
 
 
-@pytest.mark.parametrize("dtype", orc.DTYPES)
-@pytest.mark.parametrize("op", orc.OPS)
+@pytest.mark.parametrize("dtype", orc.ALL_DTYPES)
+@pytest.mark.parametrize("op", orc.OPS + (orc.AVG,))
 def test_all_reduce_every_dtype_and_op(dtype, op):
+    # the whole ncclDataType_t x {Sum, Prod, Max, Min, Avg} table; Avg is a sum divided afterwards (integers) or
+    # of inputs multiplied by 1/4 first (floats)
     check("all_reduce", dtype, op, 4, 300001, small_ints=(op == orc.PROD), seed=200 + dtype)
+
+
+@pytest.mark.parametrize("dtype", orc.FLOAT_DTYPES)
+@pytest.mark.parametrize("op", [orc.MAX, orc.MIN])
+def test_all_reduce_max_min_with_nan_operands(dtype, op):
+    # fmaxf / fminf semantics (src/include/reduce_kernel.h:344-362,442-469): the operand that is a number wins;
+    # NaN only where all four ranks hold one.  The values are compared where the oracle's result is a number.
+    from dfccl_amd.ring import VirtualRing
+    n, count = 4, 40000
+    nan_bits = {orc.F16: 0x7e00, orc.BF16: 0x7fc0}.get(dtype, np.nan)
+
+    def is_nan(x):
+        if dtype == orc.F16:
+            return np.isnan(x.view(np.float16))
+        if dtype == orc.BF16:
+            return np.isnan(orc.bf16_bits_to_f32(x))
+        return np.isnan(x)
+
+    with VirtualRing(n) as ring:
+        ring.prepare(0, "all_reduce", count, dtype, op)
+        ring.finalize()
+        sends_np = [datagen.make(dtype, 700 + r, count) for r in range(n)]
+        for x, every in zip(sends_np, (2, 3, 4, 6)):
+            x[::every] = nan_bits
+        sends = [to_gpu(dtype, x) for x in sends_np]
+        recvs = [torch.zeros(count, dtype=TORCH_OF[dtype], device=gpu_util.DEVICE) for _ in range(n)]
+        torch.cuda.current_stream().synchronize()
+        want = orc.all_reduce(dtype, op, geom_of(ring, 0), sends_np)
+        ring.run(0, sends, recvs, timeout=30)
+        nan = is_nan(want[0])
+        assert nan[::12].all() and not nan[1::12].any()
+        for r in range(n):
+            got = to_np(dtype, recvs[r])
+            assert np.array_equal(is_nan(got), nan), r
+            assert np.array_equal(got[~nan], want[r][~nan]), r
+
+
+@pytest.mark.parametrize("kind", ["reduce_scatter", "reduce"])
+@pytest.mark.parametrize("dtype", [orc.U8, orc.I64, orc.F64, orc.BF16, orc.F16])
+def test_avg_on_the_other_reducing_collectives(kind, dtype):
+    check(kind, dtype, orc.AVG, 3, 50021, root=2, seed=250 + dtype)
+
+
+@pytest.mark.parametrize("n,count", [(2, 1000), (8, 4099), (5, 100000)])
+def test_avg_small_and_ragged(n, count):
+    # 2 and 8 ranks on sizes that wave 0 folds alone, 5 ranks on 7 (odd) bytes per element boundary cases
+    check("all_reduce", orc.F32, orc.AVG, n, count, seed=260)
+    check("all_reduce", orc.I8, orc.AVG, n, count, seed=261)
+
+
+@pytest.mark.parametrize("dtype,value", [(orc.F32, 0.3), (orc.BF16, -1.5), (orc.F64, 1e-3), (orc.I32, 1000003),
+                                         (orc.U8, 3)])
+def test_premul_sum_operator(dtype, value):
+    # an operator made by ncclRedOpCreatePreMulSum: every input times the scalar (one rounding in the type), summed
+    from dfccl_amd.ring import VirtualRing
+    n, count = 4, 70001
+    bits = orc.scalar_bits(dtype, value)
+    scalar_bytes = int(bits).to_bytes(8, "little")[:orc.TYPE_SIZE[dtype]]
+    with VirtualRing(n) as ring:
+        ring.prepare(0, "all_reduce", count, dtype, premul=scalar_bytes)
+        ring.prepare(1, "reduce_scatter", count // n, dtype, premul=scalar_bytes)
+        ring.finalize()
+        sends_np, sends, recvs = make_buffers("all_reduce", dtype, n, count, 270)
+        want = orc.all_reduce(dtype, orc.PREMULSUM, geom_of(ring, 0), sends_np, scalar=bits)
+        ring.run(0, sends, recvs, timeout=30)
+        for r in range(n):
+            assert np.array_equal(to_np(dtype, recvs[r]), want[r]), r
+        rs_np, rs_send, rs_recv = make_buffers("reduce_scatter", dtype, n, count // n, 280)
+        want = orc.reduce_scatter(dtype, orc.PREMULSUM, geom_of(ring, 1), rs_np, scalar=bits)
+        ring.run(1, rs_send, rs_recv, timeout=30)
+        for r in range(n):
+            assert np.array_equal(to_np(dtype, rs_recv[r]), want[r]), r
+
+
+def test_premul_sum_operator_errors():
+    import dfccl_amd
+    from dfccl_amd import api
+    comms = api.VirtualComm.create_all(2)
+    ctxs = [api.RankCtx(r) for r in range(2)]
+    try:
+        half = np.array([0.5], np.float32).tobytes()
+        op0 = comms[0].create_premul_sum(dfccl_amd.ncclFloat32, half)
+        assert op0 >= 5
+        # an operator is tied to its datatype
+        with pytest.raises(api.NcclError) as e:
+            ctxs[0].prepare_all_reduce(100, dfccl_amd.ncclFloat16, op0, comms[0], 0)
+        assert e.value.code == 4
+        # an unknown operator value
+        with pytest.raises(api.NcclError):
+            ctxs[0].prepare_all_reduce(100, dfccl_amd.ncclFloat32, op0 + 17, comms[0], 0)
+        ctxs[0].prepare_all_reduce(100, dfccl_amd.ncclFloat32, op0, comms[0], 0)
+        # the ranks of a communicator have to agree on the scalar
+        op1 = comms[1].create_premul_sum(dfccl_amd.ncclFloat32, np.array([0.25], np.float32).tobytes())
+        with pytest.raises(api.NcclError) as e:
+            ctxs[1].prepare_all_reduce(100, dfccl_amd.ncclFloat32, op1, comms[1], 0)
+        assert e.value.code == 4
+        comms[0].destroy_op(op0)
+        with pytest.raises(api.NcclError):
+            comms[0].destroy_op(op0)
+        with pytest.raises(api.NcclError):
+            comms[0].destroy_op(dfccl_amd.ncclSum)
+    finally:
+        for c in ctxs:
+            c.destroy()
+        for c in comms:
+            c.destroy()
 
 
 @pytest.mark.parametrize("kind", ["reduce_scatter", "all_gather", "reduce", "broadcast"])
@@ -343,7 +451,13 @@ def test_prepare_validation_follows_the_reference():
             ctx.prepare_all_reduce(16, 10, api.ncclSum, comms[0], 1)  # dtype out of range
         assert e.value.code == 4
         with pytest.raises(api.NcclError) as e:
-            ctx.prepare_all_reduce(16, api.ncclFloat32, 4, comms[0], 1)  # ncclAvg is not on this path
+            ctx.prepare_all_reduce(16, api.ncclFloat32, 5, comms[0], 1)  # no operator with that value was created
+        assert e.value.code == 4
+        with pytest.raises(api.NcclError) as e:
+            ctx.prepare_all_reduce(16, api.ncclFloat32, -1, comms[0], 1)
+        assert e.value.code == 4
+        with pytest.raises(api.NcclError) as e:
+            ctx.prepare_broadcast(16, 11, 0, comms[0], 1)  # dtype out of range on a copy collective
         assert e.value.code == 4
         ctx.prepare_all_reduce(16, api.ncclFloat32, api.ncclSum, comms[0], 1)
         with pytest.raises(api.NcclError) as e:
