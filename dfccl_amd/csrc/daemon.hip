@@ -38,7 +38,10 @@
 
 namespace dfccl {
 
-constexpr int kDaemonUnroll = 1;  // see reduce_copy.hip: shallow unrolling keeps DRAM accesses ordered
+// Rows (of one 128-bit access per thread) the FIFO movers keep in flight per thread.  One: a deeper pipeline (4 rows)
+// would suit a workgroup that has its compute unit to itself and reads only two sources, but it takes the kernel
+// from 135 to 167 vector registers, and that has not been measured on a GPU yet.
+constexpr int kDaemonUnroll = 1;
 constexpr int kReadyWords = (kMaxColls + 63) / 64;
 constexpr int kSoftWaitSpins = 2;       // polls of a wait of the direct protocol while other collectives are queued
 constexpr int kSoloMaxBytes = 4096;  // largest own chunk of a one-tile collective that wave 0 runs by itself (see runDirect)

@@ -119,6 +119,7 @@ static std::unordered_map<uint64_t, CommGroup*> gGroups;
 static std::atomic<uint64_t> gNextCommId{1};
 
 struct Daemon;
+static int deviceWorkgroupSlots(int device);
 
 struct CollReg {
   int collId;
@@ -194,10 +195,7 @@ struct Daemon {
     // every workgroup of the daemon has to be resident at the same time (they wait for each other): the grid
     // may not exceed what the occupancy calculation says fits the GPU (one 512-thread workgroup per CU while
     // the kernel needs more than 128 VGPRs per lane)
-    int cus = 0, perCu = 0;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) cus = 0;
-    if (dfcclDaemonOccupancy(&perCu) != hipSuccess || perCu < 1) perCu = 1;
-    capacity = (long)cus * perCu;
+    capacity = deviceWorkgroupSlots(device);
     return capacity;
   }
 
@@ -456,6 +454,14 @@ static void destroyDaemon(Daemon* d) {
 // Rank contexts alive per device: the workgroups of all of them have to fit the GPU together.
 static std::atomic<int> gLiveRankCtxs[64];
 
+// Workgroups of the daemon kernel the device keeps resident at once (compute units x workgroups per unit).
+static int deviceWorkgroupSlots(int device) {
+  int cus = 0, perCu = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
+  if (dfcclDaemonOccupancy(&perCu) != hipSuccess || perCu < 1) perCu = 1;
+  return cus * perCu;
+}
+
 static void planGroup(CommGroup* g) {
   const int es = typeSizeOf(g->dtypeUser);
   int64_t nBytes = (int64_t)g->countUser * es;
@@ -499,12 +505,19 @@ static void planGroup(CommGroup* g) {
     g->slicesPerChunk = 2;
     g->fifoSlots = 4;
   }
-  // Default: share the 256 workgroups that fill the GPU (one per CU) among the ranks that will run together,
-  // which is the larger of this communicator's size and the rank contexts created on the device so far.
+  // Default: share the workgroups the GPU keeps resident (one per CU) among the ranks that will run together,
+  // which is the larger of this communicator's size and the rank contexts created on the device so far, and
+  // leave a few of them out (DFCCL_RESIDENCY_HEADROOM, 8): every workgroup of the daemon has to be resident,
+  // so a grid that needs every last CU would leave one workgroup waiting for a CU that another kernel's
+  // workgroup holds.  The launch rounds a rank's workgroups up to whole sets of 8 (one per XCD; the surplus
+  // ones leave at once), and that rounded grid has to fit as well.
   int sharers = g->nRanks;
   if (g->device >= 0 && g->device < 64) sharers = std::max(sharers, gLiveRankCtxs[g->device].load());
-  int share = std::max(1, 256 / std::max(1, sharers));
-  if (share > 8) share &= ~7;  // the launch rounds a rank's workgroups up to whole sets of 8 (one per XCD)
+  sharers = std::max(1, sharers);
+  const int capacity = deviceWorkgroupSlots(g->device);
+  const int headroom = (int)std::min<int64_t>(std::max<int64_t>(0, envInt("DFCCL_RESIDENCY_HEADROOM", 8)), capacity / 2);
+  int share = std::max(1, (capacity - headroom) / sharers);
+  while (share > 1 && sharers * ((share + 7) & ~7) > capacity) share--;
   int maxCh = (int)envInt("NCCL_MAX_NCHANNELS", share);
   if (maxCh < 1) maxCh = 1;
   if (maxCh > kMaxChannels) maxCh = kMaxChannels;

@@ -219,7 +219,8 @@ def test_config2_geometry_ring_all_reduce_8_ranks_bf16(proto, chunk_bytes, monke
         ring.prepare(0, "all_reduce", count, orc.BF16, orc.SUM)
         ring.finalize()
         g = ring.ctxs[0].geometry(0)
-        assert (g.nChannels == 32 or gpu_util.EMULATED) and g.protocol == (1 if proto == "direct" else 0)
+        # 8 ranks share the 256 workgroup slots less a headroom of 8: 31 channels each
+        assert (g.nChannels == 31 or gpu_util.EMULATED) and g.protocol == (1 if proto == "direct" else 0)
         if chunk_bytes is not None or proto == "fifo":
             assert g.chunkElems == 262144
         sends_np, sends, recvs = make_buffers("all_reduce", orc.BF16, n, count, 2)
