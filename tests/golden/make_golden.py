@@ -42,6 +42,20 @@ CASES = [
     ("reduce_copy", orc.BF16, orc.SUM, 3, 1000, 0, None),
     ("reduce_copy", orc.I8, orc.PROD, 4, 2000, 0, None),
     ("reduce_copy", orc.F16, orc.MAX, 8, 515, 0, None),
+    # the remaining element types and the scaled sums (appended: the cases above keep their numbers and inputs)
+    ("all_reduce", orc.U8, orc.MAX, 4, 3000, 0, (1, 8192, 1024)),
+    ("all_reduce", orc.U32, orc.SUM, 3, 1500, 0, (1, 2048, 256)),
+    ("all_reduce", orc.I64, orc.MIN, 4, 900, 0, (1, 1024, 128)),
+    ("all_reduce", orc.U64, orc.PROD, 2, 600, 0, (1, 1024, 128)),
+    ("all_reduce", orc.F64, orc.SUM, 4, 900, 0, (1, 1024, 128)),
+    ("all_reduce", orc.I32, orc.AVG, 5, 1234, 0, (1, 2048, 256)),
+    ("all_reduce", orc.U8, orc.AVG, 3, 2000, 0, (1, 8192, 1024)),
+    ("all_reduce", orc.BF16, orc.AVG, 4, 2048, 0, (1, 4096, 512)),
+    ("all_reduce", orc.F32, orc.AVG, 8, 4000, 0, (1, 2048, 256)),
+    ("reduce_scatter", orc.I64, orc.AVG, 4, 300, 0, (1, 1024, 128)),
+    ("reduce", orc.F64, orc.AVG, 3, 700, 1, (1, 1024, 128)),
+    ("reduce_copy", orc.U32, orc.AVG, 5, 1000, 0, None),
+    ("reduce_copy", orc.F16, orc.AVG, 3, 1000, 0, None),
 ]
 
 
