@@ -4,10 +4,14 @@ The file holds, for every workgroup (rank slot x channel, 16 x 64 of them), 4096
 event | arg << 32 and a 100 MHz tick; the last record slot of a workgroup holds how many records it wrote.
 
     python -m dfccl_amd.trace_summary <file> <channels per rank> [<rank slots>]
+    python -m dfccl_amd.trace_summary --steps <file> <workgroup>[,<workgroup>...]
 
 prints, for the last instance every workgroup moved data for, when (in microseconds after the first submission
 of that instance was fetched) the submissions were fetched and ingested, the data movement began and ended, the
-completions were posted and the visits ended: minimum, median and maximum over the workgroups."""
+completions were posted and the visits ended: minimum, median and maximum over the workgroups.  With --steps:
+for each of the given workgroups, every record from a fetch to the end of the visit that follows it, as
+microseconds after the fetch (median / minimum / 90th percentile over all instances with the same sequence of
+events): the step-by-step cost of one small collective."""
 import sys
 
 import numpy as np
@@ -44,7 +48,34 @@ def last_instance(records):
     return out
 
 
+def steps(path, wgs):
+    a = np.fromfile(path, dtype=np.uint64).reshape(-1, RECORDS, 2)
+    for wg in wgs:
+        n = int(a[wg, RECORDS - 1, 1])
+        rec = a[wg, :min(n, RECORDS - 1)]
+        ev = (rec[:, 0] & 0xffffffff).astype(int)
+        t = rec[:, 1].astype(np.int64)
+        seqs = {}
+        for s in np.nonzero(ev == 1)[0][5:]:  # (the first few instances are warm-up)
+            names, times = [], []
+            for j in range(s, len(ev)):
+                names.append(EVENTS.get(ev[j], str(ev[j])))
+                times.append((t[j] - t[s]) / 100.0)
+                if ev[j] == 10:
+                    break
+            seqs.setdefault(tuple(names), []).append(times)
+        print(f"workgroup {wg}: {n} records")
+        for key, v in sorted(seqs.items(), key=lambda kv: -len(kv[1]))[:2]:
+            arr = np.array(v)
+            print(f"  {len(v)} instances with this sequence (median / min / p90, us after the fetch):")
+            for i, name in enumerate(key):
+                print(f"    {name:11s} {np.median(arr[:, i]):7.2f} {arr[:, i].min():7.2f} {np.percentile(arr[:, i], 90):7.2f}")
+    return 0
+
+
 def main(argv):
+    if len(argv) > 3 and argv[1] == "--steps":
+        return steps(argv[2], [int(x) for x in argv[3].split(",")])
     path, channels = argv[1], int(argv[2])
     slots = int(argv[3]) if len(argv) > 3 else 16
     a = np.fromfile(path, dtype=np.uint64).reshape(-1, RECORDS, 2)
