@@ -436,6 +436,82 @@ def test_callback_gets_coll_id_and_args_on_poller_thread():
             c.destroy()
 
 
+@pytest.mark.parametrize("capacity,sleep_ms", [("6", 0), ("2000", 2)])
+def test_queue_back_pressure_every_submission_gets_one_callback(capacity, sleep_ms, monkeypatch):
+    # Two submitting threads per rank push 24 small all-reduces three times each as fast as Run takes them (a second
+    # Run of a collective waits for the first inside the library), the last rank starting late so that the others
+    # pile up parked collectives.  With a submission queue of 6 entries the full-queue path of Run (sqWrite
+    # returning "full", src/enqueue_ofccl.cc:623-627) and the lazily published queue head are exercised; with the
+    # full-size queue the callback sleeps on the poller thread (src/enqueue_ofccl.cc:908-965) instead.
+    import ctypes
+    import time
+    from dfccl_amd import _lib, api
+    monkeypatch.setenv("DFCCL_SQ_CAPACITY", capacity)
+    lib = _lib.load()
+    n, ncolls, rounds, count = 3, 24, 3, 600
+    comms = [api.VirtualComm.create_all(n) for _ in range(ncolls)]
+    ctxs = [api.RankCtx(r) for r in range(n)]
+    calls = [[0] * ncolls for _ in range(n)]
+    lock = threading.Lock()
+    try:
+        for c in range(ncolls):
+            for r in range(n):
+                ctxs[r].prepare_all_reduce(count, api.ncclInt32, api.ncclSum, comms[c][r], c)
+        for r in range(n):
+            ctxs[r].finalize()
+
+        @_lib.CALLBACK
+        def cb(coll_id, args):
+            if sleep_ms:
+                time.sleep(sleep_ms / 1000.0)
+            with lock:
+                calls[int(args or 0)][coll_id] += 1
+            return 0
+
+        send = [[(torch.arange(count, dtype=torch.int32) + 3 * r + 7 * c).to(gpu_util.DEVICE) for r in range(n)]
+                for c in range(ncolls)]
+        recv = [[torch.full((count,), -1, dtype=torch.int32, device=gpu_util.DEVICE) for r in range(n)]
+                for c in range(ncolls)]
+        torch.cuda.current_stream().synchronize()
+        failures = []
+
+        def submitter(r, half):
+            if r == n - 1:
+                time.sleep(0.2)
+            for _ in range(rounds):
+                for c in range(half, ncolls, 2):
+                    rc = lib.ofcclRunAllReduce(send[c][r].data_ptr(), recv[c][r].data_ptr(), c, cb,
+                                               ctypes.c_void_p(r) if r else None, ctxs[r].handle)
+                    if rc != 0:
+                        failures.append((r, c, rc))
+
+        threads = [threading.Thread(target=submitter, args=(r, h)) for r in range(n) for h in (0, 1)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(120)
+        assert not any(t.is_alive() for t in threads) and not failures
+        deadline = time.monotonic() + 60
+        while time.monotonic() < deadline and any(v < rounds for row in calls for v in row):
+            time.sleep(0.005)
+        time.sleep(0.05)  # a callback too many would show up now
+        assert all(v == rounds for row in calls for v in row), calls
+        for c in range(ncolls):
+            want = sum(torch.arange(count, dtype=torch.int32) + 3 * q + 7 * c for q in range(n))
+            for r in range(n):
+                assert torch.equal(recv[c][r].cpu(), want), (c, r)
+        stats = [ctx.stats() for ctx in ctxs]
+        assert sum(s["cqesWritten"] for s in stats) == n * ncolls * rounds
+        if int(capacity) < ncolls // 2:
+            assert sum(s["sqFullWaits"] for s in stats) > 0  # the queue really was found full
+    finally:
+        for c in ctxs:
+            c.destroy()
+        for cs in comms:
+            for c in cs:
+                c.destroy()
+
+
 def test_prepare_validation_follows_the_reference():
     from dfccl_amd import api
     comms = api.VirtualComm.create_all(2)
