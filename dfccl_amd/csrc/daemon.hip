@@ -1072,6 +1072,7 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
         ok = r.ok;
         if (ok) {
           layOutSweep(g, P, ch, inst, r.word);
+          if (tid == 0) trace(A, sh, kTrLaidOut, 0);
           if (!solo && lane == 0) {
             sh.sweep = g;  // for the other waves, and for a later visit that finds the context still resident
             sh.peersLoaded = 1;
@@ -1118,6 +1119,7 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
     } else {
       sweepFoldAny(g, sh.ticket, pos, INT64_MAX, mtid, nthr, tilesDone, finished);
       if (tid == 0) {
+        trace(A, sh, kTrFolded, 0);
         sh.progressed = 1;
         sh.stats.slicesMoved += (uint64_t)tilesDone;
       }
@@ -1231,7 +1233,9 @@ __device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgS
     trace(A, sh, kTrVisitBegin, coll);
   }
   __syncthreads();
+  if (tid == 0) trace(A, sh, kTrRunEntry, 0);
   const int status = runColl(A, sh, ch, tid);
+  if (tid == 0) trace(A, sh, kTrRunReturned, (uint32_t)status);
   __syncthreads();
   if (tid == 0) {
     if (sh.progressed) sh.progressedRound = 1;
@@ -1308,6 +1312,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
       else ingestMirror(A, R, sh, ch, lane);
       if (sh.numActive > 0) scanReady(R, sh, ch, lane);
       else if (lane == 0) sh.numReady = 0;
+      if (lane == 0 && sh.ingested > 0) trace(A, sh, kTrScanDone, 0);
       DFCCL_WAVE_LDS_SYNC();
       if (lane == 0) {
         // the host's requests and the lifetime limit are looked at every 8th round, and only every 64th while
@@ -1324,7 +1329,9 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
             sh.statsEpoch = statsReq;
             flushStats(R, sh, ch, statsReq);
           }
-          expired = K.maxLifetimeTicks > 0 && (int64_t)(wall_clock64() - startTick) > K.maxLifetimeTicks;
+          // (not in the first round of a launch: a lifetime shorter than the start-up would otherwise end every
+          // launch before its first visit, and nothing would ever move)
+          expired = K.maxLifetimeTicks > 0 && round != 0 && (int64_t)(wall_clock64() - startTick) > K.maxLifetimeTicks;
         }
         if (sh.ingested > 0 || sh.progressedRound) sh.idle = 0;
         else sh.idle++;
@@ -1359,6 +1366,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     const int numReady = sh.numReady;
     __syncthreads();
     if (roundExit != kExitNone) break;
+    if (tid == 0 && numReady > 0) trace(A, sh, kTrRoundDecided, (uint32_t)numReady);
 
     // ---- run phase: visit the collectives that can move, in arrival order
     // (traverseTaskQ, enqueue_ofccl_dev.cu:922-1016)

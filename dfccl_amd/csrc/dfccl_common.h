@@ -223,7 +223,13 @@ struct DaemonArgs {
 constexpr int kTraceRecords = 4096;
 enum TraceEvent : uint32_t {
   kTrSqeFetched = 1, kTrIngested = 2, kTrVisitBegin = 3, kTrWaitBegin = 4, kTrWaitEnd = 5, kTrMoveBegin = 6,
-  kTrMoveEnd = 7, kTrPosted = 8, kTrCqePosted = 9, kTrVisitEnd = 10, kTrScanDone = 11, kTrLaunch = 12, kTrExit = 13
+  kTrMoveEnd = 7, kTrPosted = 8, kTrCqePosted = 9, kTrVisitEnd = 10, kTrScanDone = 11, kTrLaunch = 12, kTrExit = 13,
+  // finer stamps inside one scheduler round and one visit (what the time between the events above is spent on)
+  kTrRoundDecided = 14,  // the round's decisions are taken, the run phase begins
+  kTrRunEntry = 15,      // the visit's first barrier is passed, the collective's code begins
+  kTrLaidOut = 16,       // direct protocol: sources and destinations of the sweep are known
+  kTrFolded = 17,        // direct protocol: the sweep's loads and stores are issued (before the release)
+  kTrRunReturned = 18    // the collective's code has returned to the visit
 };
 
 }  // namespace dfccl

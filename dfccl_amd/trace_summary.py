@@ -17,7 +17,8 @@ import sys
 import numpy as np
 
 EVENTS = {1: "sqeFetched", 2: "ingested", 3: "visitBegin", 4: "waitBegin", 5: "waitEnd", 6: "moveBegin", 7: "moveEnd",
-          8: "posted", 9: "cqePosted", 10: "visitEnd", 11: "scanDone", 12: "launch", 13: "exit"}
+          8: "posted", 9: "cqePosted", 10: "visitEnd", 11: "scanDone", 12: "launch", 13: "exit", 14: "roundDecided",
+          15: "runEntry", 16: "laidOut", 17: "folded", 18: "runReturned"}
 RECORDS, MAX_CHANNELS = 4096, 64
 
 

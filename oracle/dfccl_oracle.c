@@ -266,6 +266,11 @@ static void postdiv_range(int dtype, uint64_t scalar, void* x, size_t n) {
   }
 }
 
+void orc_scale_apply(int dtype, int how, uint64_t scalar, void* buf, size_t n) {
+  if (how == 1) premul_range(dtype, scalar, buf, buf, n);
+  else if (how == 2) postdiv_range(dtype, scalar, buf, n);
+}
+
 /* a rank's input as it enters the reduction: the buffer itself, or a scaled copy in tmp */
 static const void* entering(int dtype, const orc_xop* x, const void* in, void* tmp, size_t n) {
   if (!x->pre) return in;

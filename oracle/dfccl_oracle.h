@@ -84,6 +84,9 @@ int orc_reduce_copy_x(int dtype, int op, uint64_t scalar, int k, const void* con
 /* The scalar ncclAvg turns into for a group of n: n itself for integer types, 1/n rounded to the element type
  * for float types (bits in the low bytes). */
 uint64_t orc_avg_scalar(int dtype, int n);
+/* The two halves of a scaled sum on their own, in place: how = 1 multiplies every element by the scalar (one
+ * element's bits), how = 2 divides every element of an integer type by (int)scalar as SumPostDiv does. */
+void orc_scale_apply(int dtype, int how, uint64_t scalar, void* buf, size_t n);
 /* Same result, element range split statically over nthreads host threads. */
 int orc_reduce_copy_mt(int dtype, int op, int k, const void* const* srcs, void* dst, size_t n, int nthreads);
 

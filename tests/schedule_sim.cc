@@ -34,6 +34,17 @@ extern "C" int sim_collective(int kind, int dtype, int op, int n, int nChannels,
                               int64_t* maxSliceSeen) {
   const int es = (kind == kAllGather || kind == kBroadcast) ? 1 : orc_type_size(dtype);
   if (kind == kAllGather || kind == kBroadcast) { count *= orc_type_size(dtype); dtype = ORC_I8; }
+  // ncclAvg: a Sum whose user inputs are multiplied by 1/n as a step reads them (float types), or whose final
+  // value is divided by n in the step the schedule marks `post` (integer types)
+  int how = 0;
+  uint64_t scalar = 0;
+  if (op == ORC_AVG) {
+    op = ORC_SUM;
+    if (n > 1) {
+      scalar = orc_avg_scalar(dtype, n);
+      how = (dtype == ORC_F16 || dtype == ORC_BF16 || dtype == ORC_F32 || dtype == ORC_F64) ? 1 : 2;
+    }
+  }
   const int64_t real0 = realChunkElems(kind, n, nChannels, chunkElems, alignElems, count > 0 ? count : 1, 0);
   const int64_t slotElems = sliceElemsFor(real0, slicesPerChunk, sliceElems);
   *maxSliceSeen = 0;
@@ -79,9 +90,15 @@ extern "C" int sim_collective(int kind, int dtype, int op, int n, int nChannels,
               if (d.useIn) { s0 = sb + (d.inOff + off) * es; s1 = fifoIn; } else s0 = fifoIn;
               if (d.useOut) { d0 = rb + (d.outOff + off) * es; d1 = fifoOut; } else d0 = fifoOut;
               if (s0 && d0) {
-                std::vector<char> tmp((size_t)len * es);
+                std::vector<char> tmp((size_t)len * es), in0;
+                if (how == 1 && d.useIn) {  // source 0 is the user's input: scaled as it enters
+                  in0.assign(s0, s0 + (size_t)len * es);
+                  orc_scale_apply(dtype, 1, scalar, in0.data(), (size_t)len);
+                  s0 = in0.data();
+                }
                 if (s1) { const void* srcs[2] = {s0, s1}; orc_reduce_copy(dtype, op, 2, srcs, tmp.data(), (size_t)len); }
                 else memcpy(tmp.data(), s0, (size_t)len * es);
+                if (how == 2 && d.post) orc_scale_apply(dtype, 2, scalar, tmp.data(), (size_t)len);
                 memcpy(d0, tmp.data(), (size_t)len * es);
                 if (d1) memcpy(d1, tmp.data(), (size_t)len * es);
               }

@@ -52,7 +52,9 @@ CASES = [(2, 1, 64, 16, 1000), (3, 2, 64, 16, 1000), (4, 1, 128, 32, 37), (4, 3,
 
 
 @pytest.mark.parametrize("n,C,chunk,align,count", CASES)
-@pytest.mark.parametrize("dtype,op", [(orc.F32, orc.SUM), (orc.BF16, orc.SUM), (orc.I8, orc.MAX), (orc.F16, orc.PROD)])
+@pytest.mark.parametrize("dtype,op", [(orc.F32, orc.SUM), (orc.BF16, orc.SUM), (orc.I8, orc.MAX), (orc.F16, orc.PROD),
+                                      (orc.BF16, orc.AVG), (orc.I32, orc.AVG), (orc.F64, orc.AVG), (orc.U8, orc.AVG),
+                                      (orc.U64, orc.MAX)])
 def test_all_reduce_schedule_matches_oracle(sim, n, C, chunk, align, count, dtype, op):
     g = orc.Geom(n, C, chunk, align)
     sends = [datagen.make(dtype, 10 + r, count) for r in range(n)]
@@ -70,7 +72,8 @@ def test_all_reduce_schedule_matches_oracle(sim, n, C, chunk, align, count, dtyp
 
 
 @pytest.mark.parametrize("n,C,chunk,align,count", CASES)
-@pytest.mark.parametrize("dtype,op", [(orc.F32, orc.SUM), (orc.BF16, orc.MIN), (orc.I32, orc.SUM)])
+@pytest.mark.parametrize("dtype,op", [(orc.F32, orc.SUM), (orc.BF16, orc.MIN), (orc.I32, orc.SUM), (orc.F16, orc.AVG),
+                                      (orc.I64, orc.AVG)])
 def test_reduce_scatter_schedule_matches_oracle(sim, n, C, chunk, align, count, dtype, op):
     g = orc.Geom(n, C, chunk, align)
     sends = [datagen.make(dtype, 20 + r, count * n) for r in range(n)]
@@ -110,6 +113,12 @@ def test_reduce_and_broadcast_schedules_match_oracle(sim, n, C, chunk, align, co
         run_sim(sim, "reduce", orc.BF16, orc.SUM, n, C, chunk, align, chunk, 1, 8, count, root, sends, recvs)
         for r in range(n):
             assert np.array_equal(recvs[r], want[r]), (root, r)
+        for dtype in (orc.F32, orc.I8):  # an average: inputs scaled where the chain reads them, or the root divides
+            isends = [datagen.make(dtype, 45 + r, count) for r in range(n)]
+            want = orc.reduce(dtype, orc.AVG, g, root, isends)
+            recvs = [np.zeros_like(s) for s in isends]
+            run_sim(sim, "reduce", dtype, orc.AVG, n, C, chunk, align, chunk, 1, 8, count, root, isends, recvs)
+            assert np.array_equal(recvs[root], want[root]), (dtype, root)
         recvs = [np.zeros_like(s) for s in sends]
         run_sim(sim, "broadcast", orc.F16, 0, n, C, chunk, align, chunk, 1, 8, count, root, sends, recvs)
         for r in range(n):
@@ -173,7 +182,8 @@ DIRECT_CASES = [(2, 1, 64, 16, 1000), (3, 2, 64, 16, 1000), (4, 1, 128, 32, 37),
 
 @pytest.mark.parametrize("kind", list(KIND))
 @pytest.mark.parametrize("n,C,chunk,align,count", DIRECT_CASES)
-@pytest.mark.parametrize("dtype,op", [(orc.F32, orc.SUM), (orc.BF16, orc.SUM), (orc.I8, orc.MIN)])
+@pytest.mark.parametrize("dtype,op", [(orc.F32, orc.SUM), (orc.BF16, orc.SUM), (orc.I8, orc.MIN), (orc.F16, orc.AVG),
+                                      (orc.U32, orc.AVG)])
 def test_direct_protocol_roles_and_tiles_match_oracle(sim, kind, n, C, chunk, align, count, dtype, op):
     root = (n - 1) // 2
     if kind in ("reduce_scatter", "all_gather"):
