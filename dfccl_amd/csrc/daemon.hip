@@ -120,10 +120,17 @@ struct WgShared {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");  \
   } while (0)
 #endif
-// A value every lane of the wave loads from the same address with one instruction, and so gets identically;
-// lanes that run as threads of their own take lane 0's.
+// A value that has to be the same in every lane of the wave because the wave branches on it: scheduler state
+// that all lanes load from one address in LDS or global memory.  Every lane takes the first lane's copy
+// (v_readfirstlane: the value lives in scalar registers from there on and the branch is a scalar one), so the
+// lanes of a wave cannot disagree about the way to go, whatever order their loads were performed in.
 #ifndef DFCCL_WAVE_UNIFORM
-#define DFCCL_WAVE_UNIFORM(x) (x)
+__device__ __forceinline__ uint32_t waveUniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+__device__ __forceinline__ int32_t waveUniform(int32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ uint64_t waveUniform(uint64_t v) {
+  return (uint64_t)waveUniform((uint32_t)v) | ((uint64_t)waveUniform((uint32_t)(v >> 32)) << 32);
+}
+#define DFCCL_WAVE_UNIFORM(x) ::dfccl::waveUniform(x)
 #endif
 
 // Test hook of the host build: a workgroup that never leaves (it ignores the host's requests, quit entries and
@@ -242,7 +249,7 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
   // buffers named by the new entries may have been written by the host, a copy engine or another kernel
   // before the submission
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-  const int base = sh.numActive;  // (read by every lane before the ballots below, written by lane 0 after them)
+  const int base = DFCCL_WAVE_UNIFORM(sh.numActive);  // (read before the ballots below, written by lane 0 after them)
   bool isQuit = false, mine = false;
   if (lane < avail) {
     isQuit = (flags & kSqeFlagQuit) != 0;
@@ -309,7 +316,8 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
 // tag), hand them to the other channels through the HBM mirror, take them into the own task queue straight
 // from the registers, and pick up the host's control word.  (Role of sqRead, enqueue_ofccl_dev.cu:85-173.)
 __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, WgShared& sh, int lane) {
-  const uint64_t base = sh.hostFrontier;
+  const uint64_t base = DFCCL_WAVE_UNIFORM(sh.hostFrontier);
+  const int32_t numActive = DFCCL_WAVE_UNIFORM(sh.numActive);
   // With an empty task queue the leader has nothing to do but watch the ring's next entry and the control word
   // (lanes 0..3 and lane 60, one load instruction).  It keeps four such polls in flight, so that a new
   // entry is seen a fraction of a PCIe round trip after it lands rather than up to a whole one; the other
@@ -319,11 +327,11 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
   // posted fewer completions than it has fetched submissions; then the leader polls once, and rarely.
   const int idleRounds = (int)A.knobs.idlePollRounds;
   bool busy = false;
-  if (sh.numActive == 0 && R.nChannels > 1)
+  if (numActive == 0 && R.nChannels > 1)
     busy = DFCCL_WAVE_UNIFORM(__hip_atomic_load(G(R.cqTicket), __ATOMIC_RELAXED, DFCCL_AGENT)) < base;
   DFCCL_WAVE_LDS_SYNC();  // (every lane has read the state above)
   if (lane == 0) sh.rankBusy = busy ? 1 : 0;
-  const bool idleMode = sh.numActive == 0 && idleRounds > 0 && !busy;
+  const bool idleMode = numActive == 0 && idleRounds > 0 && !busy;
   const int nlanes = idleMode ? kSqeWords : kSqesPerPoll * kSqeWords;
   // every lane loads (the lanes without a word of their own re-read lane 0's, which costs nothing: it is the
   // same request), so that no load is conditional and several can stay in flight
@@ -416,15 +424,16 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
   }
   // The host may reuse entries every workgroup of the rank has consumed. It only looks at the head when the
   // ring seems full, so the head is published now and then, not on every poll.
-  if (sh.hostFrontier - sh.publishedHead >= 64 || (n == 0 && sh.hostFrontier != sh.publishedHead)) {
-    uint64_t f = sh.frontier;
+  const uint64_t fetched = DFCCL_WAVE_UNIFORM(sh.hostFrontier), published = DFCCL_WAVE_UNIFORM(sh.publishedHead);
+  if (fetched - published >= 64 || (n == 0 && fetched != published)) {
+    uint64_t f = DFCCL_WAVE_UNIFORM(sh.frontier);
     if (R.nChannels > 1) {
       f = ~0ull;
       if (lane < R.nChannels) f = __hip_atomic_load(G(&R.wgFrontier[lane]), __ATOMIC_RELAXED, DFCCL_AGENT);
       f = waveMin64(f);
     }
     DFCCL_WAVE_LDS_SYNC();
-    if (lane == 0 && f != sh.publishedHead) {
+    if (lane == 0 && f != published) {
       __hip_atomic_store(G(R.sqHead), f, __ATOMIC_RELAXED, DFCCL_SYSTEM);
       sh.publishedHead = f;
     }
@@ -434,7 +443,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
 
 // Wave 0 of the other channels: take new entries from the mirror ring, one lane per entry.
 __device__ __forceinline__ void ingestMirror(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane) {
-  const uint64_t f = sh.frontier;
+  const uint64_t f = DFCCL_WAVE_UNIFORM(sh.frontier);
   // polled with a relaxed load: an acquire would invalidate the L2 on every poll of every idle workgroup
   const uint64_t tail = DFCCL_WAVE_UNIFORM(__hip_atomic_load(G(R.mirrorTail), __ATOMIC_RELAXED, DFCCL_AGENT));
   const int avail = (int)((tail - f) < 64 ? (tail - f) : 64);
@@ -466,9 +475,9 @@ __device__ __forceinline__ bool descMet(const WaitDesc& w) {
 // Wave 0: mark the collectives of the task queue that can move, 64 per pass, one
 // lane per collective, from the wait descriptors saved with their contexts.
 __device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, int ch, int lane) {
-  const int n = sh.numActive;
+  const int n = DFCCL_WAVE_UNIFORM(sh.numActive);
   int total = 0;
-  if (sh.allFresh && sh.ingested > 0 && n <= 64) {
+  if (DFCCL_WAVE_UNIFORM(sh.allFresh) && DFCCL_WAVE_UNIFORM(sh.ingested) > 0 && n <= 64) {
     // nothing is parked: everything in the queue arrived this round and can start
     if (lane == 0) {
       sh.ready[0] = (n >= 64) ? ~0ull : ((1ull << n) - 1ull);
@@ -1310,7 +1319,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     if (wave == 0) {
       if (ch == 0) pollHost(A, R, sh, lane);
       else ingestMirror(A, R, sh, ch, lane);
-      if (sh.numActive > 0) scanReady(R, sh, ch, lane);
+      if (DFCCL_WAVE_UNIFORM(sh.numActive) > 0) scanReady(R, sh, ch, lane);
       else if (lane == 0) sh.numReady = 0;
       if (lane == 0 && sh.ingested > 0) trace(A, sh, kTrScanDone, 0);
       DFCCL_WAVE_LDS_SYNC();
@@ -1351,7 +1360,7 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
         sh.progressedRound = 0;
       }
       DFCCL_WAVE_LDS_SYNC();
-      if (sh.numReady == 0 && sh.ingested == 0) {
+      if (DFCCL_WAVE_UNIFORM(sh.numReady) == 0 && DFCCL_WAVE_UNIFORM(sh.ingested) == 0) {
         // nothing can move: the leader's next poll is a PCIe round trip anyway, the others back off a little
         if (ch != 0) __builtin_amdgcn_s_sleep(20);
         else if (sh.rankBusy) __builtin_amdgcn_s_sleep(100);
