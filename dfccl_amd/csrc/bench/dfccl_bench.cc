@@ -198,6 +198,7 @@ struct World {
       NK(dfcclGetStats(ctx[r], &s));
       t.sqesRead += s.sqesRead; t.cqesWritten += s.cqesWritten; t.ctxSaves += s.ctxSaves; t.ctxLoads += s.ctxLoads;
       t.voluntaryQuits += s.voluntaryQuits; t.forcedQuits += s.forcedQuits; t.slicesMoved += s.slicesMoved;
+      t.sqFullWaits += s.sqFullWaits;
       t.daemonLaunches = std::max(t.daemonLaunches, s.daemonLaunches);
     }
     return t;
@@ -353,10 +354,11 @@ static int runDisorder(const Args& a) {
   printf("{\"mode\": \"disorder\", \"ranks\": %d, \"colls\": %d, \"dtype\": \"%s\", \"min_bytes\": %zu, \"max_bytes\": %zu, "
          "\"total_bytes_per_rank\": %zu, \"deadlocks\": %d, \"correct\": %s, \"wall_ms\": %.3f, "
          "\"p50_us\": %.1f, \"p90_us\": %.1f, \"p99_us\": %.1f, \"small_bucket_count\": %zu, \"small_bucket_p50_us\": %.1f, "
-         "\"preemptions_ctx_saves\": %llu, \"ctx_loads\": %llu, \"cqes\": %llu}\n",
+         "\"preemptions_ctx_saves\": %llu, \"ctx_loads\": %llu, \"cqes\": %llu, \"sq_full_waits\": %llu}\n",
          n, nc, a.dtype.c_str(), a.minBytes, a.maxBytes, totalBytes, failed.load(), ok ? "true" : "false",
          (double)(tEnd.load() - t0) / 1e6, pct(all, 0.5), pct(all, 0.9), pct(all, 0.99), small.size(), pct(small, 0.5),
-         (unsigned long long)st.ctxSaves, (unsigned long long)st.ctxLoads, (unsigned long long)st.cqesWritten);
+         (unsigned long long)st.ctxSaves, (unsigned long long)st.ctxLoads, (unsigned long long)st.cqesWritten,
+         (unsigned long long)st.sqFullWaits);
   return ok ? 0 : 1;
 }
 

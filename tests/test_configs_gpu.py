@@ -35,6 +35,17 @@ def test_config3_disordered_256_collectives_no_deadlock(proto):
     assert r["cqes"] == 4 * 256
 
 
+def test_config3_disordered_with_a_submission_queue_of_four_entries():
+    # the same 256 disordered all-reduces with DFCCL_SQ_CAPACITY=4: the four submitting threads (C++, a fraction
+    # of a microsecond per Run) find the queue full over and over (certainly while the daemon is being launched),
+    # wait as ofcclRun* does in the reference (src/collectives_ofccl/ofccl_all_reduce.cc:29-33), and nothing is
+    # lost: every submission completes, every result is right
+    r = native(["disorder", "--ranks", 4, "--colls", 256, "--dtype", "fp16", "--timeout", 30], {"DFCCL_SQ_CAPACITY": "4"})
+    assert r["deadlocks"] == 0 and r["correct"] is True
+    assert r["cqes"] == 4 * 256
+    assert r["sq_full_waits"] > 0
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "int32"])
 def test_config4_gradient_buckets_full_size(dtype):
     # 4 virtual ranks, 40 buckets of 25,000,000 elements, all submitted at once; results verified element by element

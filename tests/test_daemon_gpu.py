@@ -502,8 +502,11 @@ def test_queue_back_pressure_every_submission_gets_one_callback(capacity, sleep_
                 assert torch.equal(recv[c][r].cpu(), want), (c, r)
         stats = [ctx.stats() for ctx in ctxs]
         assert sum(s["cqesWritten"] for s in stats) == n * ncolls * rounds
-        if int(capacity) < ncolls // 2:
-            assert sum(s["sqFullWaits"] for s in stats) > 0  # the queue really was found full
+        if int(capacity) < ncolls // 2 and gpu_util.EMULATED:
+            # the queue really was found full.  (Only asserted where the daemon is slow enough to make that
+            # certain: a GPU empties a queue of 6 faster than Python threads fill it, except while the kernel is
+            # being launched; there the run still checks that nothing is lost or duplicated.)
+            assert sum(s["sqFullWaits"] for s in stats) > 0
     finally:
         for c in ctxs:
             c.destroy()
