@@ -671,6 +671,47 @@ def test_other_collectives_disordered_submission(proto):
                 assert np.array_equal(to_np(orc.F32, bufs[cid][1][r]), wants[cid][r]), (cid, kind, r)
 
 
+@pytest.mark.parametrize("seed", range(int(os.environ.get("DFCCL_RANDOM_SEEDS", "8"))))  # (more for a longer campaign)
+def test_random_collectives_every_type_and_op_disordered(seed):
+    # random ranks, kinds, element types, ops (Avg included), sizes (from a few elements to several tiles, mostly
+    # ragged) and roots, registered side by side and submitted by every rank in its own order, twice
+    from dfccl_amd.ring import VirtualRing
+    rng = np.random.default_rng(9000 + seed)
+    n = int(rng.integers(2, 9))
+    ncolls = int(rng.integers(3, 8))
+    specs = []
+    for cid in range(ncolls):
+        kind = ["all_reduce", "reduce_scatter", "all_gather", "reduce", "broadcast"][int(rng.integers(5))]
+        dtype = int(rng.integers(10))
+        op = int(rng.integers(5))
+        shape = int(rng.integers(4))
+        count = [int(rng.integers(1, 17)), int(rng.integers(1, 3000)), 256 * int(rng.integers(1, 40)),
+                 int(rng.integers(1, 120000))][shape]
+        if gpu_util.EMULATED:
+            count = min(count, 30000)
+        specs.append((kind, dtype, op, count, int(rng.integers(n))))
+    with VirtualRing(n) as ring:
+        for cid, (kind, dtype, op, count, root) in enumerate(specs):
+            ring.prepare(cid, kind, count, dtype, op, root)
+        ring.finalize()
+        for rep in range(2):
+            bufs, wants = [], []
+            for cid, (kind, dtype, op, count, root) in enumerate(specs):
+                sends_np, sends, recvs = make_buffers(kind, dtype, n, count, 9100 + 100 * seed + 10 * cid + rep,
+                                                      small_ints=(op == orc.PROD))
+                bufs.append((sends, recvs))
+                wants.append(oracle_run(kind, dtype, op, geom_of(ring, cid), root, sends_np))
+            for r in range(n):
+                for cid in rng.permutation(ncolls):
+                    ring.submit(r, int(cid), bufs[cid][0][r], bufs[cid][1][r])
+            ring.wait([(r, cid) for r in range(n) for cid in range(ncolls)], timeout=60)
+            for cid, (kind, dtype, op, count, root) in enumerate(specs):
+                for r in range(n):
+                    if kind == "reduce" and r != root:
+                        continue
+                    assert np.array_equal(to_np(dtype, bufs[cid][1][r]), wants[cid][r]), (seed, rep, cid, specs[cid], r)
+
+
 @pytest.mark.parametrize("knobs", [{"BASE_CTX_SWITCH_THRESHOLD": "1", "NUM_TRY_TASKQ_HEAD": "1", "RECV_SUCCESS_FACTOR": "0"},
                                    {}, {"DFCCL_IDLE_POLL_ROUNDS": "0"}])
 def test_small_all_reduce_repeated_and_fallbacks(knobs, monkeypatch):
