@@ -9,7 +9,7 @@
 //   emul_stress mixed <ranks> <reps>    all five collectives side by side, int32, ranks submit in different orders
 //   emul_stress relaunch <ranks>        idle exit and relaunch, with and without a collective parked
 //   emul_stress reuse <ranks>           rank contexts destroyed and created again: old communicators are refused
-//   emul_stress fuzz <seed> <rounds>    random collectives, ranks and submission orders
+//   emul_stress fuzz <seed> <rounds>    random collectives, element types, ops, ranks and submission orders
 //   emul_stress backpressure <ranks> <colls> <rounds> <callback sleep us>   two submitting threads per rank push
 //        every collective `rounds` times as fast as the queue takes them (DFCCL_SQ_CAPACITY makes it small), the
 //        last rank starting late; every submission must get exactly one callback
@@ -101,9 +101,19 @@ static T* devAlloc(size_t count) {
   gBuffers.push_back(p);
   return (T*)p;
 }
+static std::vector<char*> gExactBuffers;
+// Host memory of exactly `bytes` bytes (16-byte aligned), standing in for device memory: AddressSanitizer then
+// reports the first byte a kernel touches past the end, which hipMalloc's rounding would hide.
+static char* exactAlloc(size_t bytes) {
+  char* p = new char[bytes ? bytes : 1];
+  gExactBuffers.push_back(p);
+  return p;
+}
 static void freeBuffers() {
   for (void* p : gBuffers) hipFree(p);
   gBuffers.clear();
+  for (char* p : gExactBuffers) delete[] p;
+  gExactBuffers.clear();
 }
 
 static uint16_t bf16Of(int v) {  // small integers are exact in bfloat16
@@ -357,8 +367,38 @@ static int scenarioReuse(int n) {
   return 0;
 }
 
-// Random collectives (kind, count, root), every rank submits them in its own random order, several rounds; int32
-// Sum so that any result can be checked exactly.  The knobs come from the environment.
+// One small non-negative integer as an element of any ncclDataType_t (exact in every type up to 2048).
+static int elemSize(int dt) {
+  switch (dt) {
+    case ncclInt8: case ncclUint8: return 1;
+    case ncclFloat16: case ncclBfloat16: return 2;
+    case ncclInt32: case ncclUint32: case ncclFloat32: return 4;
+    default: return 8;
+  }
+}
+static void putElem(void* base, size_t i, int dt, int v) {
+  char* p = (char*)base + i * (size_t)elemSize(dt);
+  switch (dt) {
+    case ncclInt8: case ncclUint8: { uint8_t x = (uint8_t)v; memcpy(p, &x, 1); break; }
+    case ncclInt32: case ncclUint32: { int32_t x = v; memcpy(p, &x, 4); break; }
+    case ncclInt64: case ncclUint64: { int64_t x = v; memcpy(p, &x, 8); break; }
+    case ncclFloat16: { _Float16 x = (_Float16)v; memcpy(p, &x, 2); break; }
+    case ncclBfloat16: { uint16_t x = bf16Of(v); memcpy(p, &x, 2); break; }
+    case ncclFloat32: { float x = (float)v; memcpy(p, &x, 4); break; }
+    default: { double x = (double)v; memcpy(p, &x, 8); break; }
+  }
+}
+static bool elemIs(const void* base, size_t i, int dt, int v) {
+  char want[8], got[8];
+  putElem(want, 0, dt, v);
+  memcpy(got, (const char*)base + i * (size_t)elemSize(dt), (size_t)elemSize(dt));
+  return memcmp(want, got, (size_t)elemSize(dt)) == 0;
+}
+
+// Random collectives (kind, count, root, element type, op), every rank submits them in its own random order,
+// several rounds.  Inputs are small non-negative integers, so that Sum, Max and the integer Avg have exact
+// results in every element type and any result can be checked with integer arithmetic.  The knobs come from the
+// environment.
 static int scenarioFuzz(uint64_t seed, int rounds) {
   uint64_t x = seed * 0x9e3779b97f4a7c15ull + 12345;
   auto rnd = [&](uint64_t m) {
@@ -368,7 +408,7 @@ static int scenarioFuzz(uint64_t seed, int rounds) {
     return (x >> 11) % m;
   };
   const int n = 2 + (int)rnd(5), ncolls = 1 + (int)rnd(7);
-  struct Coll { int kind, count, root; };
+  struct Coll { int kind, count, root, dt, op; };
   std::vector<Coll> colls;
   Ring ring(n);
   for (int c = 0; c < ncolls; c++) {
@@ -377,34 +417,56 @@ static int scenarioFuzz(uint64_t seed, int rounds) {
     const int shape = (int)rnd(4);
     k.count = shape == 0 ? 1 + (int)rnd(16) : shape == 1 ? 1 + (int)rnd(3000) : shape == 2 ? 256 * (1 + (int)rnd(40)) : 1 + (int)rnd(60000);
     k.root = (int)rnd((uint64_t)n);
+    k.dt = (int)rnd(10);
+    const bool isFloat = k.dt == ncclFloat16 || k.dt == ncclFloat32 || k.dt == ncclFloat64 || k.dt == ncclBfloat16;
+    const int pick = (int)rnd(3);
+    k.op = pick == 0 ? (int)ncclSum : pick == 1 ? (int)ncclMax : (isFloat ? (int)ncclMin : (int)ncclAvg);
     colls.push_back(k);
     auto& comms = ring.newComms();
+    const ncclDataType_t dt = (ncclDataType_t)k.dt;
+    const ncclRedOp_t op = (ncclRedOp_t)k.op;
     for (int r = 0; r < n; r++) {
       switch (k.kind) {
-        case 0: CHECK(ofcclPrepareAllReduce(k.count, ncclInt32, ncclSum, comms[r], c, ring.ctxs[r])); break;
-        case 1: CHECK(ofcclPrepareReduceScatter(k.count, ncclInt32, ncclSum, comms[r], c, ring.ctxs[r])); break;
-        case 2: CHECK(ofcclPrepareAllGather(k.count, ncclInt32, comms[r], c, ring.ctxs[r])); break;
-        case 3: CHECK(ofcclPrepareReduce(k.count, ncclInt32, ncclSum, k.root, comms[r], c, ring.ctxs[r])); break;
-        default: CHECK(ofcclPrepareBroadcast(k.count, ncclInt32, k.root, comms[r], c, ring.ctxs[r])); break;
+        case 0: CHECK(ofcclPrepareAllReduce(k.count, dt, op, comms[r], c, ring.ctxs[r])); break;
+        case 1: CHECK(ofcclPrepareReduceScatter(k.count, dt, op, comms[r], c, ring.ctxs[r])); break;
+        case 2: CHECK(ofcclPrepareAllGather(k.count, dt, comms[r], c, ring.ctxs[r])); break;
+        case 3: CHECK(ofcclPrepareReduce(k.count, dt, op, k.root, comms[r], c, ring.ctxs[r])); break;
+        default: CHECK(ofcclPrepareBroadcast(k.count, dt, k.root, comms[r], c, ring.ctxs[r])); break;
       }
     }
   }
   ring.finalize();
   auto sendLen = [&](int c) { return colls[c].kind == 1 ? colls[c].count * n : colls[c].count; };
   auto recvLen = [&](int c) { return colls[c].kind == 2 ? colls[c].count * n : colls[c].count; };
-  std::vector<std::vector<int32_t*>> send((size_t)ncolls), recv((size_t)ncolls);
+  std::vector<std::vector<char*>> send((size_t)ncolls), recv((size_t)ncolls);
   for (int c = 0; c < ncolls; c++)
     for (int r = 0; r < n; r++) {
-      send[c].push_back(devAlloc<int32_t>((size_t)sendLen(c)));
-      recv[c].push_back(devAlloc<int32_t>((size_t)recvLen(c)));
+      // (exactly as long as the collective needs: an access past the end is AddressSanitizer's to report)
+      send[c].push_back(exactAlloc((size_t)sendLen(c) * elemSize(colls[c].dt)));
+      recv[c].push_back(exactAlloc((size_t)recvLen(c) * elemSize(colls[c].dt)));
     }
-  auto val = [](int c, int r, int i, int rep) { return (int32_t)(i * 31 + r * 1009 + c * 77 + rep * 5); };
+  auto val = [](int c, int r, int i, int rep) { return (i * 31 + r * 5 + c * 7 + rep * 3) % 4; };
+  auto reduce = [&](int c, int i, int rep) {  // the reduction of element i over the ranks
+    int acc = 0, mx = 0, mn = 1 << 30;
+    for (int q = 0; q < n; q++) {
+      const int v = val(c, q, i, rep);
+      acc += v;
+      mx = v > mx ? v : mx;
+      mn = v < mn ? v : mn;
+    }
+    switch (colls[c].op) {
+      case ncclSum: return acc;
+      case ncclMax: return mx;
+      case ncclMin: return mn;
+      default: return acc / n;  // ncclAvg of an integer type
+    }
+  };
   std::vector<int> want((size_t)n * ncolls, 0);
   for (int rep = 0; rep < rounds; rep++) {
     for (int c = 0; c < ncolls; c++)
       for (int r = 0; r < n; r++) {
-        for (int i = 0; i < sendLen(c); i++) send[c][r][i] = val(c, r, i, rep);
-        for (int i = 0; i < recvLen(c); i++) recv[c][r][i] = -7;
+        for (int i = 0; i < sendLen(c); i++) putElem(send[c][r], (size_t)i, colls[c].dt, val(c, r, i, rep));
+        memset(recv[c][r], 0x5a, (size_t)recvLen(c) * elemSize(colls[c].dt));
       }
     // per-rank random order; ranks are interleaved at random as well
     std::vector<std::vector<int>> order((size_t)n);
@@ -435,15 +497,15 @@ static int scenarioFuzz(uint64_t seed, int rounds) {
         const int kind = colls[c].kind, count = colls[c].count, root = colls[c].root;
         if (kind == 3 && r != root) continue;
         for (int i = 0; i < recvLen(c); i++) {
-          int32_t e = 0;
-          if (kind == 0 || kind == 3) for (int q = 0; q < n; q++) e += val(c, q, i, rep);
-          else if (kind == 1) for (int q = 0; q < n; q++) e += val(c, q, r * count + i, rep);
+          int e;
+          if (kind == 0 || kind == 3) e = reduce(c, i, rep);
+          else if (kind == 1) e = reduce(c, r * count + i, rep);
           else if (kind == 2) e = val(c, i / count, i % count, rep);
           else e = val(c, root, i, rep);
-          if (recv[c][r][i] != e) {
-            fprintf(stderr, "emul_stress: fuzz seed %llu: round %d collective %d (kind %d, count %d, root %d) rank %d of %d "
-                    "element %d: %d, expected %d\n", (unsigned long long)seed, rep, c, kind, count, root, r, n, i,
-                    recv[c][r][i], e);
+          if (!elemIs(recv[c][r], (size_t)i, colls[c].dt, e)) {
+            fprintf(stderr, "emul_stress: fuzz seed %llu: round %d collective %d (kind %d, type %d, op %d, count %d, root %d) "
+                    "rank %d of %d element %d: expected %d\n", (unsigned long long)seed, rep, c, kind, colls[c].dt,
+                    colls[c].op, count, root, r, n, i, e);
             return 1;
           }
         }
