@@ -175,9 +175,13 @@ ncclResult_t ofcclRunAllGather(const void* sendbuff, void* recvbuff, int collId,
  * (src/include/common_kernel.h:557-622,629-690).  The same device code moves
  * the data inside the daemon kernel; this entry point exposes it for the
  * semantics check against a host loop and for the bandwidth measurement.
- * srcs is a host array of nsrcs (1..8) device pointers; chunkBytes is the
+ * Every ncclDataType_t; op is Sum, Prod, Max, Min or Avg (the average over
+ * the nsrcs sources: integer sums divided by nsrcs afterwards, float inputs
+ * multiplied by 1/nsrcs first, as ncclAvg over nsrcs ranks would be).
+ * srcs is a host array of nsrcs (1..8) device pointers; more than four
+ * sources take several launches that fold into dst.  chunkBytes is the
  * grain handed to one workgroup at a time (0 = default); stream is a
- * hipStream_t (NULL = the null stream).  Asynchronous. */
+ * hipStream_t (NULL = the null stream).  Asynchronous; allocates nothing. */
 ncclResult_t dfcclReduceCopy(const void* const* srcs, int nsrcs, void* dst, size_t count, ncclDataType_t datatype,
                              ncclRedOp_t op, size_t chunkBytes, void* stream);
 
