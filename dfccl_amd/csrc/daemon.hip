@@ -40,7 +40,7 @@ namespace dfccl {
 
 // Rows (of one 128-bit access per thread) the FIFO movers keep in flight per thread.  One: a deeper pipeline (4 rows)
 // would suit a workgroup that has its compute unit to itself and reads only two sources, but it takes the kernel
-// from 135 to 167 vector registers, and that has not been measured on a GPU yet.
+// to about 170 vector registers, and that has not been measured on a GPU yet.
 constexpr int kDaemonUnroll = 1;
 constexpr int kReadyWords = (kMaxColls + 63) / 64;
 constexpr int kSoftWaitSpins = 2;       // polls of a wait of the direct protocol while other collectives are queued
