@@ -222,8 +222,11 @@ __device__ __forceinline__ void reportStuck(const RankDev& R, WgShared& sh, int 
   const uint32_t coll = sh.taskq[0];
   if (coll >= (uint32_t)R.nColls) return;
   DynCtx d;
-  if ((int32_t)coll == sh.loadedColl) d = sh.dyn;
-  else loadStruct(d, &R.dyn[(size_t)ch * R.nColls + coll]);
+  if ((int32_t)coll == sh.loadedColl) {
+    d = sh.dyn;
+  } else {
+    loadStruct(d, &R.dyn[(size_t)ch * R.nColls + coll]);
+  }
   uint64_t seen = 0;
   if ((d.wait[0].count & (kWaitTagged - 1)) > 0)
     seen = __hip_atomic_load((const DFCCL_GLOBAL uint64_t*)(uintptr_t)d.wait[0].ptr, __ATOMIC_RELAXED, DFCCL_AGENT);
@@ -336,8 +339,11 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
   // every lane loads (the lanes without a word of their own re-read lane 0's, which costs nothing: it is the
   // same request), so that no load is conditional and several can stay in flight
   const uint64_t* pw = R.sq + ((base & (kSqRing - 1)) * kSqeWords);
-  if (lane < nlanes) pw = R.sq + (((base + (uint64_t)(lane >> 2)) & (kSqRing - 1)) * kSqeWords + (lane & 3));
-  else if (lane == 60) pw = (const uint64_t*)R.ctrl;  // the control word's allocation is 64 bytes long
+  if (lane < nlanes) {
+    pw = R.sq + (((base + (uint64_t)(lane >> 2)) & (kSqRing - 1)) * kSqeWords + (lane & 3));
+  } else if (lane == 60) {
+    pw = (const uint64_t*)R.ctrl;  // the control word's allocation is 64 bytes long
+  }
   const DFCCL_GLOBAL uint64_t* p = (const DFCCL_GLOBAL uint64_t*)pw;
   const uint64_t tagWant = sqeTag(base + (uint64_t)(lane >> 2));
   uint64_t w;
@@ -804,9 +810,13 @@ __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, 
 template <int DT, int OP, bool SC = false>
 __device__ __forceinline__ void sweepFold(const SweepGeom& g, uint64_t* slots, int64_t& pos, int64_t maxTiles, int tid,
                                           int nthr, int64_t& tilesDone, bool& finished) {
-  if (g.n <= 2) sweepFoldN<DT, OP, 2, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
-  else if (g.n <= 4) sweepFoldN<DT, OP, 4, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
-  else sweepFoldN<DT, OP, 8, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
+  if (g.n <= 2) {
+    sweepFoldN<DT, OP, 2, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
+  } else if (g.n <= 4) {
+    sweepFoldN<DT, OP, 4, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
+  } else {
+    sweepFoldN<DT, OP, 8, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
+  }
 }
 
 template <int DT>
@@ -853,8 +863,11 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
   char* sendFifo = P.sendFifo + (int64_t)ch * P.fifoChanStride;
   const char* recvFifo = P.recvFifo + (int64_t)ch * P.fifoChanStride;
   int inPlace;
-  if (kind == kAllGather) inPlace = (sendbuff == recvbuff + (int64_t)P.rank * count * es);
-  else inPlace = (sendbuff == recvbuff);
+  if (kind == kAllGather) {
+    inPlace = (sendbuff == recvbuff + (int64_t)P.rank * count * es);
+  } else {
+    inPlace = (sendbuff == recvbuff);
+  }
 
   int64_t grid = sh.dyn.gridOffset;
   int step0 = sh.dyn.step, slice0 = sh.dyn.slice;
@@ -897,10 +910,18 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
         void* d1 = nullptr;
         const void* fifoIn = d.recv ? recvFifo + (int64_t)(recvStep % (uint64_t)P.fifoSlots) * P.slotBytes : nullptr;
         void* fifoOut = d.send ? sendFifo + (int64_t)(sendStep % (uint64_t)P.fifoSlots) * P.slotBytes : nullptr;
-        if (d.useIn) { s0 = sendbuff + (d.inOff + off) * es; s1 = fifoIn; }
-        else s0 = fifoIn;
-        if (d.useOut) { d0 = recvbuff + (d.outOff + off) * es; d1 = fifoOut; }
-        else d0 = fifoOut;
+        if (d.useIn) {
+          s0 = sendbuff + (d.inOff + off) * es;
+          s1 = fifoIn;
+        } else {
+          s0 = fifoIn;
+        }
+        if (d.useOut) {
+          d0 = recvbuff + (d.outOff + off) * es;
+          d1 = fifoOut;
+        } else {
+          d0 = fifoOut;
+        }
         if (s0 != nullptr && d0 != nullptr) {
           // a scaled sum (ncclAvg / PreMulSum) multiplies the user's input where it enters (source 0 of a step that
           // reads it) and divides where the final value is produced
@@ -1057,8 +1078,11 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
   // nothing is held while parked), and the workgroup is better off moving the next collective's data.
   const int64_t cap = (sh.numActive > 1 && forceEvery == 0) ? kSoftWaitSpins : 0;
   // every thread has taken its copy of the position before thread 0 changes it
-  if (solo) DFCCL_WAVE_LDS_SYNC();
-  else __syncthreads();
+  if (solo) {
+    DFCCL_WAVE_LDS_SYNC();
+  } else {
+    __syncthreads();
+  }
 
   if (!published && tid < 2) {
     // the words carry their own instance tag: no ordering between them is needed, and the buffers' contents
@@ -1136,8 +1160,11 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
     // Released to the system here, while the peers are still busy, so that the completion need not wait for it.
     // Whole workgroup: the barrier orders every thread's stores before thread 0's fence.  Wave 0 alone: every
     // lane's stores are covered by the fence the wave executes together.
-    if (solo) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-    else __syncthreads();
+    if (solo) {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+    } else {
+      __syncthreads();
+    }
     if (tid == 0) {
       trace(A, sh, kTrMoveEnd, 0);
       if (!solo) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
@@ -1206,8 +1233,11 @@ __device__ __forceinline__ void completeColl(const DaemonArgs& A, const RankDev&
     const uint64_t t = (R.nChannels == 1) ? sh.cqNext++
                                           : __hip_atomic_fetch_add(G(R.cqTicket), 1ull, __ATOMIC_RELAXED, DFCCL_AGENT);
     const uint64_t cqe = cqeEncode((unsigned)ch, (unsigned)(t + 1), (unsigned)sh.plan.collId);
-    if (sh.released) __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]), cqe, __ATOMIC_RELAXED, DFCCL_SYSTEM);
-    else __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]), cqe, __ATOMIC_RELEASE, DFCCL_SYSTEM);
+    if (sh.released) {
+      __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]), cqe, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+    } else {
+      __hip_atomic_store(G(&R.cq[t & (kCqRing - 1)]), cqe, __ATOMIC_RELEASE, DFCCL_SYSTEM);
+    }
     sh.stats.cqesWritten++;
     trace(A, sh, kTrCqePosted, coll);
   }
@@ -1317,11 +1347,19 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
   for (;;) {
     // ---- ingest phase (wave 0)
     if (wave == 0) {
-      if (ch == 0) pollHost(A, R, sh, lane);
-      else ingestMirror(A, R, sh, ch, lane);
-      if (DFCCL_WAVE_UNIFORM(sh.numActive) > 0) scanReady(R, sh, ch, lane);
-      else if (lane == 0) sh.numReady = 0;
-      if (lane == 0 && sh.ingested > 0) trace(A, sh, kTrScanDone, 0);
+      if (ch == 0) {
+        pollHost(A, R, sh, lane);
+      } else {
+        ingestMirror(A, R, sh, ch, lane);
+      }
+      if (DFCCL_WAVE_UNIFORM(sh.numActive) > 0) {
+        scanReady(R, sh, ch, lane);
+      } else if (lane == 0) {
+        sh.numReady = 0;
+      }
+      if (lane == 0 && sh.ingested > 0) {
+        trace(A, sh, kTrScanDone, 0);
+      }
       DFCCL_WAVE_LDS_SYNC();
       if (lane == 0) {
         // the host's requests and the lifetime limit are looked at every 8th round, and only every 64th while
@@ -1342,13 +1380,19 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
           // launch before its first visit, and nothing would ever move)
           expired = K.maxLifetimeTicks > 0 && round != 0 && (int64_t)(wall_clock64() - startTick) > K.maxLifetimeTicks;
         }
-        if (sh.ingested > 0 || sh.progressedRound) sh.idle = 0;
-        else sh.idle++;
+        if (sh.ingested > 0 || sh.progressedRound) {
+          sh.idle = 0;
+        } else {
+          sh.idle++;
+        }
         if (sh.numActive > 0 && sh.idle > 0 && (sh.idle & (kStuckReportRounds - 1)) == 0) reportStuck(R, sh, ch);
-        if (abortFlag) sh.exitKind = kExitAbort;
-        else if (sh.finalQuit) sh.exitKind = kExitFinal;
-        else if (quitFlag || expired) sh.exitKind = kExitVoluntary;
-        else if (sh.idle >= K.tolerantUnprogressedCnt) {
+        if (abortFlag) {
+          sh.exitKind = kExitAbort;
+        } else if (sh.finalQuit) {
+          sh.exitKind = kExitFinal;
+        } else if (quitFlag || expired) {
+          sh.exitKind = kExitVoluntary;
+        } else if (sh.idle >= K.tolerantUnprogressedCnt) {
           // Idle for long: leave, and take the whole daemon along (every workgroup saves its state and leaves at
           // its next look at this flag).  The kernel can only be launched again once all of it has ended, and a
           // submission for a rank whose workgroups have left is not seen by anybody until then: a daemon that
@@ -1362,8 +1406,11 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
       DFCCL_WAVE_LDS_SYNC();
       if (DFCCL_WAVE_UNIFORM(sh.numReady) == 0 && DFCCL_WAVE_UNIFORM(sh.ingested) == 0) {
         // nothing can move: the leader's next poll is a PCIe round trip anyway, the others back off a little
-        if (ch != 0) __builtin_amdgcn_s_sleep(20);
-        else if (sh.rankBusy) __builtin_amdgcn_s_sleep(100);
+        if (ch != 0) {
+          __builtin_amdgcn_s_sleep(20);
+        } else if (sh.rankBusy) {
+          __builtin_amdgcn_s_sleep(100);
+        }
       }
     }
     __syncthreads();

@@ -31,9 +31,11 @@
  * per-element closed form of the ring order for the schedules, permutation
  * identities for the copy collectives).  Not pinned by anything but a live run
  * of the reference, and therefore judged by invariants only: which collectives
- * get preempted and the order of completions.  Max/Min on NaN or on +0 vs -0
- * is "parity unpinned" (implementation-defined in the reference's intrinsics);
- * test inputs avoid both.
+ * get preempted and the order of completions.  Max/Min with NaN operands
+ * follow fmaxf / fminf (the operand that is a number wins) and are pinned
+ * against float64 extremes over the non-NaN operands.  Which of +0 and -0
+ * Max/Min return is "parity unpinned" (not fixed by fmax / fmin); test inputs
+ * avoid mixing the two zeros.
  */
 #ifndef DFCCL_ORACLE_H_
 #define DFCCL_ORACLE_H_
