@@ -26,6 +26,7 @@ sys.path.insert(0, os.path.join(ROOT, "oracle"))
 
 HBM_PEAK_GBPS = 8000.0
 PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "reduce_copy_f32_sum_k2_256MiB.md")
+DAEMON_PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "daemon_all_reduce_8x64MiB_bf16_pmc.md")
 
 
 def measured_traffic_bytes():
@@ -36,6 +37,18 @@ def measured_traffic_bytes():
     try:
         with open(PROFILE_SUMMARY) as f:
             m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", f.read(), re.M)
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def measured_daemon_traffic_bytes(label):
+    """HBM bytes one 8 x 64 MiB bf16 all-reduce moved through the daemon under rocprofv3 --pmc (line
+    `traffic_bytes_per_all_reduce_<label>:` of the daemon's profile summary).  None if no such run is recorded."""
+    import re
+    try:
+        with open(DAEMON_PROFILE_SUMMARY) as f:
+            m = re.search(r"^traffic_bytes_per_all_reduce_%s:\s*(\d+)" % re.escape(label), f.read(), re.M)
         return int(m.group(1)) if m else None
     except OSError:
         return None
@@ -155,7 +168,8 @@ def daemon_roofline(ar):
     for label, alg in (("direct", 2 * n * nbytes), ("fifo_512KiB_chunks", (6 * n - 4) * nbytes)):
         ms = ar[label]["ms"]
         gbps = alg / (ms * 1e-3) / 1e9
-        out[label] = {"bytes": alg, "ms": ms, "achieved": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+        out[label] = {"bytes": alg, "ms": ms, "achieved": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                      "traffic": measured_daemon_traffic_bytes(label.split("_")[0])}
     return out
 
 
@@ -174,7 +188,11 @@ def bench_disordered():
     r = run_native(["disorder", "--ranks", 4, "--colls", 256, "--dtype", "fp16"])
     return {"workload": "256 all-reduces, 4 virtual ranks, sizes log-uniform 4 KiB..4 MiB fp16, per-rank random order",
             "deadlocks": r["deadlocks"], "correct": r["correct"], "wall_ms": r["wall_ms"], "p50_us": r["p50_us"],
-            "p99_us": r["p99_us"], "preemptions": r["preemptions_ctx_saves"], "completions": r["cqes"]}
+            "p99_us": r["p99_us"],
+            # the latency this configuration is quoted on: SQE->CQE p50 of its smallest collectives (4..8 KiB),
+            # submitted among all the others in every rank's own order
+            "small_bucket_p50_us": r["small_bucket_p50_us"], "small_bucket_count": r["small_bucket_count"],
+            "preemptions": r["preemptions_ctx_saves"], "completions": r["cqes"]}
 
 
 def bench_buckets():
@@ -246,17 +264,25 @@ def main():
         "frac_of_hbm_peak": round(gbps_wall / HBM_PEAK_GBPS, 4),
         "roofline": {"bound": "hbm", "achieved": round(gbps_kernel, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4), "traffic": measured_traffic_bytes(),
-                     "kernel": "reduceCopyKernel<f32,Sum,2>", "kernel_ms_avg": round(rc["kernel_ms_avg"], 5),
+                     "kernel": "reduceCopyKernel<7,0,2,false> (fp32, Sum, 2 sources, unscaled)", "kernel_ms_avg": round(rc["kernel_ms_avg"], 5),
                      "kernel_ms_min": round(rc["kernel_ms_min"], 5),
                      "kernel_ms_avg_each_launch_bracketed_by_events": round(rc["kernel_ms_avg_bracketed"], 5)},
     }
     if not args.skip_daemon:
-        line["daemon_all_reduce"] = bench_daemon_all_reduce()
-        line["daemon_roofline"] = daemon_roofline(line["daemon_all_reduce"])
-        line["sqe_to_cqe_latency"] = bench_latency()
-        line["disordered_small_collectives"] = bench_disordered()
-        line["gradient_buckets"] = bench_buckets()
-        line["other_collectives"] = bench_other_collectives()
+        # (a leg that fails is reported as such: the headline above does not depend on it)
+        def leg(name, fn, *a):
+            try:
+                line[name] = fn(*a)
+            except Exception as e:  # noqa: BLE001
+                line[name] = {"error": f"{type(e).__name__}: {e}"[:500]}
+                print(f"bench.py: {name} failed: {e}", file=sys.stderr)
+        leg("daemon_all_reduce", bench_daemon_all_reduce)
+        if "error" not in line["daemon_all_reduce"]:
+            leg("daemon_roofline", daemon_roofline, line["daemon_all_reduce"])
+        leg("sqe_to_cqe_latency", bench_latency)
+        leg("disordered_small_collectives", bench_disordered)
+        leg("gradient_buckets", bench_buckets)
+        leg("other_collectives", bench_other_collectives)
     if not args.skip_cpu:
         line["cpu_baseline"] = bench_cpu_baseline()
     print(json.dumps(line))

@@ -19,7 +19,7 @@ class UniqueId(ctypes.Structure):
 
 class Stats(ctypes.Structure):
     _fields_ = [(n, ctypes.c_uint64) for n in
-                ("sqesRead", "cqesWritten", "ctxSaves", "ctxLoads", "voluntaryQuits", "daemonLaunches",
+                ("structBytes", "sqesRead", "cqesWritten", "ctxSaves", "ctxLoads", "voluntaryQuits", "daemonLaunches",
                  "forcedQuits", "slicesMoved", "sqFullWaits")]
 
 

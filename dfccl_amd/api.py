@@ -87,9 +87,15 @@ class VirtualComm:
         uid = cls.unique_id()
         return [cls(nranks, uid, r) for r in range(nranks)]
 
-    def create_premul_sum(self, dtype, scalar_bytes):
-        """ncclRedOpCreatePreMulSum with the scalar given as the bytes of one element; returns the op value."""
+    def create_premul_sum(self, dtype, scalar_bytes=None, device_ptr=None):
+        """ncclRedOpCreatePreMulSum; returns the op value.  The scalar is given as the bytes of one element
+        (ncclScalarHostImmediate), or as the device address it is to be read from whenever an instance starts
+        (ncclScalarDevice)."""
         op = ctypes.c_int()
+        if device_ptr is not None:
+            check(_lib.load().ncclRedOpCreatePreMulSum(ctypes.byref(op), ctypes.c_void_p(device_ptr), dtype,
+                                                       ncclScalarDevice, self.handle), "ncclRedOpCreatePreMulSum")
+            return op.value
         buf = ctypes.create_string_buffer(bytes(scalar_bytes).ljust(8, b"\0"), 8)
         check(_lib.load().ncclRedOpCreatePreMulSum(ctypes.byref(op), ctypes.cast(buf, ctypes.c_void_p), dtype,
                                                    ncclScalarHostImmediate, self.handle), "ncclRedOpCreatePreMulSum")
@@ -189,6 +195,7 @@ class RankCtx:
 
     def stats(self):
         s = Stats()
+        s.structBytes = ctypes.sizeof(Stats)
         check(self.lib.dfcclGetStats(self.handle, ctypes.byref(s)), "dfcclGetStats")
         return {n: getattr(s, n) for n, _ in Stats._fields_}
 

@@ -195,6 +195,7 @@ struct World {
     dfcclStats t{};
     for (int r = 0; r < n; r++) {
       dfcclStats s{};
+      s.structBytes = sizeof(s);
       NK(dfcclGetStats(ctx[r], &s));
       t.sqesRead += s.sqesRead; t.cqesWritten += s.cqesWritten; t.ctxSaves += s.ctxSaves; t.ctxLoads += s.ctxLoads;
       t.voluntaryQuits += s.voluntaryQuits; t.forcedQuits += s.forcedQuits; t.slicesMoved += s.slicesMoved;
@@ -208,6 +209,7 @@ struct World {
     (void)dfcclDumpState(ctx[0]);
     for (int r = 0; r < n; r++) {
       dfcclStats s{};
+      s.structBytes = sizeof(s);
       if (dfcclGetStats(ctx[r], &s) != ncclSuccess) continue;
       fprintf(stderr, "rank %d: sqes read %llu, cqes written %llu, ctx saves %llu, loads %llu, slices moved %llu, "
               "voluntary quits %llu, launches %llu\n", r, (unsigned long long)s.sqesRead,

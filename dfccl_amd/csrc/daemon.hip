@@ -36,12 +36,34 @@
 #include "dfccl_common.h"
 #include "reduce_copy_wg.h"
 
+// This file is compiled twice: as it is (the kernel that normally runs), and with DFCCL_TRACED_BUILD defined, which
+// adds the timeline stamps and gives the kernel and its launcher names of their own; the runtime launches the
+// traced kernel when DFCCL_TRACE=1 asks for a timeline.
+#ifdef DFCCL_TRACED_BUILD
+#define DFCCL_DAEMON_KERNEL dfcclDaemonKernelTraced
+#define DFCCL_DAEMON_LAUNCH dfcclLaunchDaemonTraced
+#define DFCCL_DAEMON_OCCUPANCY dfcclDaemonOccupancyTraced
+#else
+#define DFCCL_DAEMON_KERNEL dfcclDaemonKernel
+#define DFCCL_DAEMON_LAUNCH dfcclLaunchDaemon
+#define DFCCL_DAEMON_OCCUPANCY dfcclDaemonOccupancy
+#endif
+
 namespace dfccl {
 
-// Rows (of one 128-bit access per thread) the FIFO movers keep in flight per thread.  One: a deeper pipeline (4 rows)
-// would suit a workgroup that has its compute unit to itself and reads only two sources, but it takes the kernel
-// to about 170 vector registers, and that has not been measured on a GPU yet.
-constexpr int kDaemonUnroll = 1;
+#ifdef DFCCL_TRACED_BUILD
+constexpr bool kTracedBuild = true;
+#else
+constexpr bool kTracedBuild = false;
+#endif
+
+// Rows (of one 128-bit access per thread) the FIFO movers keep in flight per thread and source.  A daemon
+// workgroup has its compute unit to itself and a FIFO step reads at most two sources, so one row would leave
+// 16 KiB in flight per compute unit, half of what the one-shot reduce-copy kernel keeps there with its two
+// workgroups; two rows match it.  The movers of scaled sums keep one row (their integer divisions need the
+// registers), and the kernel's register count is bounded by a test of the compiler's resource remarks.
+constexpr int kFifoUnroll = 2;
+constexpr int kFifoUnrollScaled = 1;
 constexpr int kReadyWords = (kMaxColls + 63) / 64;
 constexpr int kSoftWaitSpins = 2;       // polls of a wait of the direct protocol while other collectives are queued
 constexpr int kSoloMaxBytes = 4096;  // largest own chunk of a one-tile collective that wave 0 runs by itself (see runDirect)
@@ -58,31 +80,41 @@ struct SweepGeom {
   int n, C, ch, es;                  // n: sources folded (1 = plain copy)
   int me, dtype, op, nd;             // nd: destinations written
   int tn, tme, scaleKind, pad1;      // a loop holds C * tn chunks, mine is number tme of every channel slot
-  uint64_t scaleBits;                // scaled sums: see Scale in reduce_ops.h
+  uint64_t scaleBits;                // scaled sums (see Scale in reduce_ops.h): the divisor of kScalePost
   uint64_t src[kMaxDirectRanks];     // the send buffers in fold order: in[me + 1], in[me + 2], ..., in[me]
   uint64_t dst[kMaxDirectRanks];     // every rank's receive buffer
 };
-struct WgShared {
-  // scheduler state
+// Scheduler state that only wave 0 uses, kept in registers: every lane of wave 0 holds the same values (they come
+// from ballots and from loads that all lanes make of one address) and applies the same updates to them, so none
+// of it goes through LDS, where every step of one lane's bookkeeping was a round trip of its own.  (The other
+// waves carry a copy that nobody looks at.)
+struct Wave0Regs {
   uint64_t frontier;       // next submission ticket this workgroup reads from the mirror ring
   uint64_t hostFrontier;   // leader: next ticket to fetch from the host ring (== mirror tail)
   uint64_t publishedHead;  // leader: last value written to the host's head word
   int64_t idle;            // consecutive rounds without work or progress
+  uint32_t round;          // scheduler rounds since launch
+  uint32_t statsReqSeen;   // leader: last request number passed on to the other workgroups
+  int32_t numActive;       // this round's copy of the task queue's length (LDS holds it for the other waves)
+  int32_t ingested;        // entries taken from the submission queue this round
+  int32_t allFresh;        // every collective of the task queue was ingested this round (nothing is parked)
+  int32_t rankBusy;        // leader: other channels of the rank still have work in flight
+  int32_t finalQuit;       // a quit entry has been read
+  int32_t numReady;        // collectives that can move this round
+};
+
+struct WgShared {
+  // scheduler state the waves share
   int32_t numActive;
   int32_t numReady;
-  int32_t finalQuit;
   int32_t exitKind;
-  int32_t ingested;
   int32_t progressedRound;
   int32_t loadedColl;      // collective whose plan and position are in LDS, -1: none
   uint32_t statsEpoch;     // last request for the counters this workgroup has answered
-  uint32_t statsReqSeen;   // leader: last request number passed on to the other workgroups
   uint32_t traceCount;
   uint32_t wgIndex;
-  uint32_t round;          // scheduler rounds since launch
-  int32_t rankBusy;        // leader: other channels of the rank still have work in flight
-  int32_t allFresh;        // every collective of the task queue was ingested this round (nothing is parked)
   uint64_t cqNext;         // single-channel ranks: next completion ticket
+  Wave0Regs w0;            // wave 0's registers, set aside while the workgroup moves data (see the run phase)
   // collective being run
   int32_t waitOk;
   int32_t progressed;
@@ -93,11 +125,17 @@ struct WgShared {
   DynCtx dyn;
   WgStats stats;
   SweepGeom sweep;         // arguments of the direct protocol's sweeps
+  uint64_t sweepScale[kMaxDirectRanks];  // pre-multiplied sums: the scalar that belongs to sweep.src[t] (see runDirect)
   uint64_t ticket[2];      // tile numbers handed from thread 0 to the workgroup (two slots, used alternately)
   uint64_t ready[kReadyWords];
+  uint64_t readySolo[kReadyWords];  // those of `ready` that wave 0 runs alone (see visit)
   uint16_t taskq[kMaxColls];
-  uint8_t collChannels[kMaxColls];  // channels of every collective of this rank (copied from the plans at launch)
+  // of every collective of this rank (from the plans, at launch): its channels in the low bits, kCollSolo if
+  // wave 0 runs it alone
+  uint8_t collChannels[kMaxColls];
 };
+constexpr uint8_t kCollSolo = 0x80;
+static_assert(kMaxChannels < kCollSolo, "the channel count shares a byte with the flag");
 
 // the workgroup's one LDS object (a host build that emulates workgroups with threads supplies its own definition)
 #ifndef DFCCL_WG_SHARED
@@ -130,7 +168,34 @@ __device__ __forceinline__ int32_t waveUniform(int32_t v) { return __builtin_amd
 __device__ __forceinline__ uint64_t waveUniform(uint64_t v) {
   return (uint64_t)waveUniform((uint32_t)v) | ((uint64_t)waveUniform((uint32_t)(v >> 32)) << 32);
 }
+__device__ __forceinline__ int64_t waveUniform(int64_t v) { return (int64_t)waveUniform((uint64_t)v); }
+template <typename T>
+__device__ __forceinline__ T* waveUniform(T* p) {
+  return (T*)(uintptr_t)waveUniform((uint64_t)(uintptr_t)p);
+}
 #define DFCCL_WAVE_UNIFORM(x) ::dfccl::waveUniform(x)
+#endif
+// A value that IS the same in every lane of the wave by construction: read from LDS after a barrier of the
+// workgroup, or computed from such values.  Everything read from LDS arrives in vector registers, and the
+// compiler cannot know that all lanes hold the same: it would keep the whole state of the scheduler and of the
+// running collective (dozens of counters, sizes and pointers) once per lane, and treat every branch on them as
+// divergent.  Taking lane 0's copy tells it: the value lives in scalar registers from there on (64 of them fit
+// one vector register when they have to be set aside), and the branch is a scalar one.  Only at places that
+// all lanes of the wave reach together.  (A host build that runs every lane as a thread checks that the lanes do
+// hold the same value.)
+#ifndef DFCCL_UNIFORM
+#define DFCCL_UNIFORM(x) ::dfccl::waveUniform(x)
+#endif
+
+// The scheduler is one endless loop with all of the data movement inlined into it.  Left alone, the compiler
+// moves everything that does not change from round to round out of that loop: every expression in the thread
+// number (lane masks, byte offsets of the thread's packs, comparisons of the lane with constants, for each of
+// the inlined movers) is computed once at the kernel's entry and then kept in registers for the kernel's whole
+// life, dozens of vector registers and as many scalar pairs that are live across everything.  Passing the
+// thread number through an empty asm statement at the head of every round makes it a new value per round as far
+// as the compiler can tell, so those expressions are computed where they are used and die there.
+#ifndef DFCCL_FRESH_PER_ROUND
+#define DFCCL_FRESH_PER_ROUND(v) asm volatile("" : "+v"(v))
 #endif
 
 // Test hook of the host build: a workgroup that never leaves (it ignores the host's requests, quit entries and
@@ -193,8 +258,38 @@ __device__ __forceinline__ WaitDesc waitFor(const void* ptr, uint64_t value, int
   return w;
 }
 
-// One record of the optional timeline (one thread per workgroup calls this).
+// The scalar of a PreMulSum operator that lives in device memory: one element of `es` bytes, read afresh
+// (the caller may have written it with a copy or a kernel since the previous instance).
+__device__ __forceinline__ uint64_t loadScalar(const void* p, int es) {
+  switch (es) {
+    case 1: return __hip_atomic_load((const DFCCL_GLOBAL uint8_t*)p, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+    case 2: return __hip_atomic_load((const DFCCL_GLOBAL uint16_t*)p, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+    case 4: return __hip_atomic_load((const DFCCL_GLOBAL uint32_t*)p, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+    default: return __hip_atomic_load((const DFCCL_GLOBAL uint64_t*)p, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+  }
+}
+
+// One thread: tell the peers where this rank's buffers of instance `inst` of a direct collective are.  The two
+// words carry their own instance tag, so no ordering between them is needed, and the buffers' contents were
+// made visible by whoever wrote them before the submission.  A scalar in device memory (scalePtr) is read now
+// and handed over with the buffers: it has to be visible to whoever sees the tags, hence the release.
+__device__ __forceinline__ void publishBuffers(PeerPub* myPub, uint64_t sendbuff, uint64_t recvbuff, uint64_t inst,
+                                               const void* scalePtr, int elemSize) {
+  const uint64_t tag = pubTag(inst);
+  if (scalePtr != nullptr) {
+    __hip_atomic_store(G(&myPub->scale), loadScalar(scalePtr, elemSize), __ATOMIC_RELAXED, DFCCL_AGENT);
+    __hip_atomic_store(G(&myPub->send), sendbuff | tag, __ATOMIC_RELEASE, DFCCL_AGENT);
+    __hip_atomic_store(G(&myPub->recv), recvbuff | tag, __ATOMIC_RELEASE, DFCCL_AGENT);
+  } else {
+    __hip_atomic_store(G(&myPub->send), sendbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
+    __hip_atomic_store(G(&myPub->recv), recvbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
+  }
+}
+
+// One record of the optional timeline (one thread per workgroup calls this).  The stamps are only compiled into
+// the traced build of this file (see kTracedBuild): the kernel that runs otherwise carries none of it.
 __device__ __forceinline__ void trace(const DaemonArgs& A, WgShared& sh, uint32_t ev, uint32_t arg) {
+  if constexpr (!kTracedBuild) return;
   if (A.trace == nullptr) return;
   const uint32_t i = sh.traceCount++;
   DFCCL_GLOBAL uint64_t* rec = G(A.trace) + ((size_t)sh.wgIndex * kTraceRecords + (i % kTraceRecords)) * 2;
@@ -246,17 +341,17 @@ __device__ __forceinline__ void reportStuck(const RankDev& R, WgShared& sh, int 
 
 // Wave 0: append the entries held one per lane (lanes < avail) to the task queue if this channel takes part
 // in them; a quit entry ends the batch.  (Role of checkSQ7TidyTaskQ, enqueue_ofccl_dev.cu:491-627.)
-__device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane,
-                                              int avail, uint64_t sendbuff, uint64_t recvbuff, uint32_t coll,
+__device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev& R, WgShared& sh, Wave0Regs& st, int ch,
+                                              int lane, int avail, uint64_t sendbuff, uint64_t recvbuff, uint32_t coll,
                                               uint32_t flags) {
   // buffers named by the new entries may have been written by the host, a copy engine or another kernel
   // before the submission
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-  const int base = DFCCL_WAVE_UNIFORM(sh.numActive);  // (read before the ballots below, written by lane 0 after them)
+  const int base = st.numActive;
   bool isQuit = false, mine = false;
   if (lane < avail) {
     isQuit = (flags & kSqeFlagQuit) != 0;
-    if (!isQuit && coll < (uint32_t)R.nColls) mine = ch < (int)sh.collChannels[coll];
+    if (!isQuit && coll < (uint32_t)R.nColls) mine = ch < (int)(sh.collChannels[coll] & (kCollSolo - 1));
   }
   const uint64_t qm = __ballot(isQuit);
   const int q = qm ? (int)__builtin_ctzll(qm) : 64;
@@ -276,10 +371,8 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
       sh.peersLoaded = 0;
       if (sh.plan.proto == kProtoDirect && sh.dyn.slice == 0) {
         // and tell the peers at once where its buffers are, instead of when the scheduler gets to it
-        PeerPub* myPub = &sh.plan.pubs[(size_t)sh.plan.rank * sh.plan.nChannels + ch];
-        const uint64_t tag = pubTag(sh.dyn.instance);
-        __hip_atomic_store(G(&myPub->send), sendbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
-        __hip_atomic_store(G(&myPub->recv), recvbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
+        publishBuffers(&sh.plan.pubs[(size_t)sh.plan.rank * sh.plan.nChannels + ch], sendbuff, recvbuff,
+                       sh.dyn.instance, sh.plan.scalePtr, sh.plan.elemSize);
         sh.dyn.slice = 1;
       }
     } else {
@@ -290,37 +383,36 @@ __device__ __forceinline__ void ingestEntries(const DaemonArgs& A, const RankDev
       const DFCCL_GLOBAL CollPlan* pl = G(&R.plans[coll]);
       if (pl->proto == kProtoDirect &&
           __hip_atomic_load(G(&d->slice), __ATOMIC_RELAXED, DFCCL_AGENT) == 0) {
-        const uint64_t tag = pubTag(__hip_atomic_load(G(&d->instance), __ATOMIC_RELAXED, DFCCL_AGENT));
-        PeerPub* myPub = &pl->pubs[(size_t)pl->rank * pl->nChannels + ch];
-        __hip_atomic_store(G(&myPub->send), sendbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
-        __hip_atomic_store(G(&myPub->recv), recvbuff | tag, __ATOMIC_RELAXED, DFCCL_AGENT);
+        publishBuffers(&pl->pubs[(size_t)pl->rank * pl->nChannels + ch], sendbuff, recvbuff,
+                       __hip_atomic_load(G(&d->instance), __ATOMIC_RELAXED, DFCCL_AGENT), pl->scalePtr, pl->elemSize);
         d->slice = 1;
       }
     }
     sh.taskq[base + pos] = (uint16_t)coll;
   }
+  int added = __builtin_popcountll(mm);
+  if (added > kMaxColls - base) added = kMaxColls - base;  // (only the entries that were stored above)
+  const int consumed = take + (q < avail ? 1 : 0);
+  st.numActive = base + added;
+  st.frontier += (uint64_t)consumed;
+  if (q < avail) st.finalQuit = 1;
+  st.ingested = consumed;
+  st.allFresh = (base == 0) ? 1 : 0;
   if (lane == 0) {
-    int added = __builtin_popcountll(mm);
-    if (added > kMaxColls - base) added = kMaxColls - base;  // (only the entries that were stored above)
     sh.numActive = base + added;
-    const int consumed = take + (q < avail ? 1 : 0);
-    sh.frontier += (uint64_t)consumed;
-    if (q < avail) sh.finalQuit = 1;
-    sh.ingested = consumed;
-    sh.allFresh = (base == 0) ? 1 : 0;
     sh.stats.sqesRead += (uint64_t)consumed;
-    if (R.nChannels > 1) __hip_atomic_store(G(&R.wgFrontier[ch]), sh.frontier, __ATOMIC_RELAXED, DFCCL_AGENT);
+    if (R.nChannels > 1) __hip_atomic_store(G(&R.wgFrontier[ch]), st.frontier, __ATOMIC_RELAXED, DFCCL_AGENT);
     trace(A, sh, kTrIngested, (uint32_t)consumed);
   }
-  DFCCL_WAVE_LDS_SYNC();
+  DFCCL_WAVE_LDS_SYNC();  // (the lanes' task queue entries are in place before any lane reads the queue)
 }
 
 // Leader, wave 0: fetch submissions from the host ring (four lanes per entry, each word validated by its own
 // tag), hand them to the other channels through the HBM mirror, take them into the own task queue straight
 // from the registers, and pick up the host's control word.  (Role of sqRead, enqueue_ofccl_dev.cu:85-173.)
-__device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, WgShared& sh, int lane) {
-  const uint64_t base = DFCCL_WAVE_UNIFORM(sh.hostFrontier);
-  const int32_t numActive = DFCCL_WAVE_UNIFORM(sh.numActive);
+__device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, WgShared& sh, Wave0Regs& st, int lane) {
+  const uint64_t base = st.hostFrontier;
+  const int32_t numActive = st.numActive;
   // With an empty task queue the leader has nothing to do but watch the ring's next entry and the control word
   // (lanes 0..3 and lane 60, one load instruction).  It keeps four such polls in flight, so that a new
   // entry is seen a fraction of a PCIe round trip after it lands rather than up to a whole one; the other
@@ -332,8 +424,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
   bool busy = false;
   if (numActive == 0 && R.nChannels > 1)
     busy = DFCCL_WAVE_UNIFORM(__hip_atomic_load(G(R.cqTicket), __ATOMIC_RELAXED, DFCCL_AGENT)) < base;
-  DFCCL_WAVE_LDS_SYNC();  // (every lane has read the state above)
-  if (lane == 0) sh.rankBusy = busy ? 1 : 0;
+  st.rankBusy = busy ? 1 : 0;
   const bool idleMode = numActive == 0 && idleRounds > 0 && !busy;
   const int nlanes = idleMode ? kSqeWords : kSqesPerPoll * kSqeWords;
   // every lane loads (the lanes without a word of their own re-read lane 0's, which costs nothing: it is the
@@ -379,14 +470,14 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
       DFCCL_IDLE_STEP(q3)
     }
 #undef DFCCL_IDLE_STEP
-    if (lane == 0 && polls > 1) sh.idle += polls - 1;
+    if (polls > 1) st.idle += polls - 1;  // (the same count in every lane: the loop ends on a ballot)
   }
   const bool valid = lane < nlanes && (w & ~kPtrMask) == tagWant;
   const uint64_t ctrlWord = __shfl(w, 60);
   const uint32_t ctrl = (uint32_t)ctrlWord, statsReq = (uint32_t)(ctrlWord >> 32);
-  if (lane == 0 && statsReq != sh.statsReqSeen) {
-    sh.statsReqSeen = statsReq;
-    __hip_atomic_store(G(&A.devFlags[2]), statsReq, __ATOMIC_RELAXED, DFCCL_AGENT);
+  if (statsReq != st.statsReqSeen) {
+    st.statsReqSeen = statsReq;
+    if (lane == 0) __hip_atomic_store(G(&A.devFlags[2]), statsReq, __ATOMIC_RELAXED, DFCCL_AGENT);
   }
   if (ctrl != 0 && lane == 0) {
     if (ctrl & kCtrlQuitRequest) __hip_atomic_store(G(&A.devFlags[0]), 1u, __ATOMIC_RELAXED, DFCCL_AGENT);
@@ -396,8 +487,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
   int n = 0;
   while (n < kSqesPerPoll && ((vm >> (4 * n)) & 0xfull) == 0xfull) n++;
   if (n == 0) {
-    if (lane == 0) sh.ingested = 0;
-    DFCCL_WAVE_LDS_SYNC();
+    st.ingested = 0;
   } else {
     // lane k < n takes entry k
     const int srcLane = (lane * 4) & 63;
@@ -421,41 +511,36 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
       DFCCL_WAVE_LDS_SYNC();  // (the wave's fence covers all its lanes' stores)
       if (lane == 0) __hip_atomic_store(G(R.mirrorTail), base + (uint64_t)n, __ATOMIC_RELAXED, DFCCL_AGENT);
     }
-    if (lane == 0) {
-      sh.hostFrontier = base + (uint64_t)n;
-      trace(A, sh, kTrSqeFetched, (uint32_t)n);
-    }
-    DFCCL_WAVE_LDS_SYNC();
-    ingestEntries(A, R, sh, 0, lane, n, sendbuff, recvbuff, coll, flags);
+    st.hostFrontier = base + (uint64_t)n;
+    if (lane == 0) trace(A, sh, kTrSqeFetched, (uint32_t)n);
+    ingestEntries(A, R, sh, st, 0, lane, n, sendbuff, recvbuff, coll, flags);
   }
   // The host may reuse entries every workgroup of the rank has consumed. It only looks at the head when the
   // ring seems full, so the head is published now and then, not on every poll.
-  const uint64_t fetched = DFCCL_WAVE_UNIFORM(sh.hostFrontier), published = DFCCL_WAVE_UNIFORM(sh.publishedHead);
+  const uint64_t fetched = st.hostFrontier, published = st.publishedHead;
   if (fetched - published >= 64 || (n == 0 && fetched != published)) {
-    uint64_t f = DFCCL_WAVE_UNIFORM(sh.frontier);
+    uint64_t f = st.frontier;
     if (R.nChannels > 1) {
       f = ~0ull;
       if (lane < R.nChannels) f = __hip_atomic_load(G(&R.wgFrontier[lane]), __ATOMIC_RELAXED, DFCCL_AGENT);
       f = waveMin64(f);
     }
-    DFCCL_WAVE_LDS_SYNC();
-    if (lane == 0 && f != published) {
-      __hip_atomic_store(G(R.sqHead), f, __ATOMIC_RELAXED, DFCCL_SYSTEM);
-      sh.publishedHead = f;
+    if (f != published) {
+      if (lane == 0) __hip_atomic_store(G(R.sqHead), f, __ATOMIC_RELAXED, DFCCL_SYSTEM);
+      st.publishedHead = f;
     }
-    DFCCL_WAVE_LDS_SYNC();
   }
 }
 
 // Wave 0 of the other channels: take new entries from the mirror ring, one lane per entry.
-__device__ __forceinline__ void ingestMirror(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int lane) {
-  const uint64_t f = DFCCL_WAVE_UNIFORM(sh.frontier);
+__device__ __forceinline__ void ingestMirror(const DaemonArgs& A, const RankDev& R, WgShared& sh, Wave0Regs& st, int ch,
+                                             int lane) {
+  const uint64_t f = st.frontier;
   // polled with a relaxed load: an acquire would invalidate the L2 on every poll of every idle workgroup
   const uint64_t tail = DFCCL_WAVE_UNIFORM(__hip_atomic_load(G(R.mirrorTail), __ATOMIC_RELAXED, DFCCL_AGENT));
   const int avail = (int)((tail - f) < 64 ? (tail - f) : 64);
   if (avail <= 0) {
-    if (lane == 0) sh.ingested = 0;
-    DFCCL_WAVE_LDS_SYNC();
+    st.ingested = 0;
     return;
   }
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -464,7 +549,7 @@ __device__ __forceinline__ void ingestMirror(const DaemonArgs& A, const RankDev&
   e.coll = 0;
   e.flags = 0;
   if (lane < avail) loadStruct(e, &R.mirror[(f + (uint64_t)lane) & (kSqRing - 1)]);
-  ingestEntries(A, R, sh, ch, lane, avail, e.sendbuff, e.recvbuff, e.coll, e.flags);
+  ingestEntries(A, R, sh, st, ch, lane, avail, e.sendbuff, e.recvbuff, e.coll, e.flags);
 }
 
 // One lane: is this parked collective's wait condition met?
@@ -479,35 +564,41 @@ __device__ __forceinline__ bool descMet(const WaitDesc& w) {
 }
 
 // Wave 0: mark the collectives of the task queue that can move, 64 per pass, one
-// lane per collective, from the wait descriptors saved with their contexts.
-__device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, int ch, int lane) {
-  const int n = DFCCL_WAVE_UNIFORM(sh.numActive);
-  int total = 0;
-  if (DFCCL_WAVE_UNIFORM(sh.allFresh) && DFCCL_WAVE_UNIFORM(sh.ingested) > 0 && n <= 64) {
-    // nothing is parked: everything in the queue arrived this round and can start
-    if (lane == 0) {
-      sh.ready[0] = (n >= 64) ? ~0ull : ((1ull << n) - 1ull);
-      sh.numReady = n;
-    }
-    DFCCL_WAVE_LDS_SYNC();
+// lane per collective, from the wait descriptors saved with their contexts; and which of them wave 0 runs alone.
+__device__ __forceinline__ void scanReady(const RankDev& R, WgShared& sh, Wave0Regs& st, int ch, int lane) {
+  const int n = st.numActive;
+  if (n == 0) {
+    st.numReady = 0;
+    if (lane == 0) sh.numReady = 0;
     return;
   }
+  const bool fresh = st.allFresh && st.ingested > 0 && n <= 64;  // nothing is parked: everything arrived this round
+  int total = 0;
   for (int base = 0; base < n; base += 64) {
     const int i = base + lane;
-    bool ready = false;
+    bool ready = false, solo = false;
     if (i < n) {
-      WaitDesc w0, w1;
-      const DynCtx* d = &R.dyn[(size_t)ch * R.nColls + sh.taskq[i]];
-      loadStruct(w0, &d->wait[0]);
-      loadStruct(w1, &d->wait[1]);
-      ready = descMet(w0) && descMet(w1);
+      const uint32_t coll = sh.taskq[i];
+      solo = (sh.collChannels[coll] & kCollSolo) != 0;
+      if (fresh) {
+        ready = true;
+      } else {
+        WaitDesc w0, w1;
+        const DynCtx* d = &R.dyn[(size_t)ch * R.nColls + coll];
+        loadStruct(w0, &d->wait[0]);
+        loadStruct(w1, &d->wait[1]);
+        ready = descMet(w0) && descMet(w1);
+      }
     }
-    const uint64_t m = __ballot(ready);
-    if (lane == 0) sh.ready[base >> 6] = m;
+    const uint64_t m = __ballot(ready), ms = __ballot(ready && solo);
+    if (lane == 0) {
+      sh.ready[base >> 6] = m;
+      sh.readySolo[base >> 6] = ms;
+    }
     total += __builtin_popcountll(m);
   }
+  st.numReady = total;
   if (lane == 0) sh.numReady = total;
-  DFCCL_WAVE_LDS_SYNC();
 }
 
 // Outcome of a bounded wait.  `ok` comes from a ballot, so every lane of the wave holds the same value in a
@@ -585,10 +676,10 @@ __device__ __forceinline__ void moveReduce(const void* s0, const void* s1, void*
   const void* s[2] = {s0, s1};
   if (d1 != nullptr) {
     void* d[2] = {d0, d1};
-    reduceCopyWG<DT, OP, 2, 2, kDaemonUnroll, false>(s, d, nbytes, tid, kWgThreads);
+    reduceCopyWG<DT, OP, 2, 2, kFifoUnroll, true, false, false>(s, d, nbytes, tid, kWgThreads);
   } else {
     void* d[1] = {d0};
-    reduceCopyWG<DT, OP, 2, 1, kDaemonUnroll, false>(s, d, nbytes, tid, kWgThreads);
+    reduceCopyWG<DT, OP, 2, 1, kFifoUnroll, true, false, false>(s, d, nbytes, tid, kWgThreads);
   }
 }
 
@@ -607,10 +698,10 @@ __device__ __forceinline__ void copySlice(const void* s0, void* d0, void* d1, si
   const void* s[1] = {s0};
   if (d1 != nullptr) {
     void* d[2] = {d0, d1};
-    reduceCopyWG<kI8, kSum, 1, 2, kDaemonUnroll, false>(s, d, nbytes, tid, kWgThreads);
+    reduceCopyWG<kI8, kSum, 1, 2, kFifoUnroll, true, false, false>(s, d, nbytes, tid, kWgThreads);
   } else {
     void* d[1] = {d0};
-    reduceCopyWG<kI8, kSum, 1, 1, kDaemonUnroll, false>(s, d, nbytes, tid, kWgThreads);
+    reduceCopyWG<kI8, kSum, 1, 1, kFifoUnroll, true, false, false>(s, d, nbytes, tid, kWgThreads);
   }
 }
 
@@ -648,19 +739,19 @@ __device__ __forceinline__ void moveScaled(const void* s0, const void* s1, void*
     const void* s[2] = {s0, s1};
     if (d1 != nullptr) {
       void* d[2] = {d0, d1};
-      reduceCopyWG<DT, kSum, 2, 2, kDaemonUnroll, false, true>(s, d, nbytes, tid, kWgThreads, su);
+      reduceCopyWG<DT, kSum, 2, 2, kFifoUnrollScaled, true, true, false>(s, d, nbytes, tid, kWgThreads, su);
     } else {
       void* d[1] = {d0};
-      reduceCopyWG<DT, kSum, 2, 1, kDaemonUnroll, false, true>(s, d, nbytes, tid, kWgThreads, su);
+      reduceCopyWG<DT, kSum, 2, 1, kFifoUnrollScaled, true, true, false>(s, d, nbytes, tid, kWgThreads, su);
     }
   } else {
     const void* s[1] = {s0};
     if (d1 != nullptr) {
       void* d[2] = {d0, d1};
-      reduceCopyWG<DT, kSum, 1, 2, kDaemonUnroll, false, true>(s, d, nbytes, tid, kWgThreads, su);
+      reduceCopyWG<DT, kSum, 1, 2, kFifoUnrollScaled, true, true, false>(s, d, nbytes, tid, kWgThreads, su);
     } else {
       void* d[1] = {d0};
-      reduceCopyWG<DT, kSum, 1, 1, kDaemonUnroll, false, true>(s, d, nbytes, tid, kWgThreads, su);
+      reduceCopyWG<DT, kSum, 1, 1, kFifoUnrollScaled, true, true, false>(s, d, nbytes, tid, kWgThreads, su);
     }
   }
 }
@@ -670,6 +761,13 @@ __device__ __forceinline__ void moveSliceScaled(int dtype, const void* s0, const
 }
 
 // Direct protocol data movement.  A "tile" is one rank's chunk of one loop.
+
+// The value lane `srcLane` of the wave holds (srcLane is the same in every lane): a register read, no LDS.
+__device__ __forceinline__ uint64_t readLane64(uint64_t v, int srcLane) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, srcLane);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), srcLane);
+  return (uint64_t)lo | ((uint64_t)hi << 32);
+}
 
 __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
@@ -683,17 +781,24 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
 // re-read src[0] (they hit in cache) so that every array element is defined: predicated loads made the compiler
 // keep the packs in scratch.  A destination may be one of the sources (in place): each thread reads a pack
 // before it writes it, and no other thread touches that pack.
-// SC: a scaled sum (OP is kSum): every source is a user input and is multiplied by the scalar first (kScalePre), or
-// the result is divided by the group size (kScalePost, integer types).
+// SC: a scaled sum (OP is kSum): every source is a user input and is multiplied by its rank's scalar first
+// (kScalePre; lane j of `scaleV` holds the scalar that belongs to src[j]), or the result is divided by the group
+// size (kScalePost, integer types).
 template <int DT, int OP, int NS, bool SC = false>
 __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks], const uint64_t (&dst)[kMaxDirectRanks],
                                          int n, int nd, int64_t byteOff, size_t nbytes, int tid, int nthr,
-                                         int scaleKind = kScaleNone, uint64_t scaleBits = 0) {
+                                         int scaleKind, uint64_t scaleV, uint64_t scaleBits) {
   constexpr int ES = typeSize(DT);
   const bool pre = SC && scaleKind == kScalePre;
   const bool post = SC && !isFloatType(DT) && scaleKind == kScalePost;
-  const u32x4 factor = splatScalar<DT>(scaleBits);
   const int divisor = (int)scaleBits;
+  // lane j of every wave holds the scalar that belongs to src[j] (all lanes are here: the call is uniform)
+  uint64_t scale[NS];
+#pragma unroll
+  for (int j = 0; j < NS; j++) {
+    if constexpr (SC) scale[j] = readLane64(scaleV, j);
+    else scale[j] = 0;
+  }
   uint64_t align = (uint64_t)byteOff;
 #pragma unroll
   for (int j = 0; j < NS; j++) align |= (j < n ? src[j] : 0);
@@ -709,7 +814,7 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
       for (int j = 0; j < NS; j++) v[j] = loadPack<true>((const char*)(j < n ? src[j] : src[0]) + byteOff, i);
       if (pre) {
 #pragma unroll
-        for (int j = 0; j < NS; j++) v[j] = packOp<DT, kProd>(v[j], factor);
+        for (int j = 0; j < NS; j++) v[j] = packOp<DT, kProd>(v[j], splatScalar<DT>(scale[j]));
       }
       u32x4 acc = v[0];
 #pragma unroll
@@ -726,12 +831,12 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
 #pragma clang loop vectorize(disable) interleave(disable) unroll(disable)
   for (size_t i = first + tid; i < nelem; i += nthr) {
     uint64_t acc = loadElem<ES>((const char*)src[0] + byteOff, i);
-    if (pre) acc = elemPreMul<DT>(acc, scaleBits);
+    if (pre) acc = elemPreMul<DT>(acc, scale[0]);
 #pragma unroll
     for (int j = 1; j < NS; j++)
       if (j < n) {
         uint64_t v = loadElem<ES>((const char*)src[j] + byteOff, i);
-        if (pre) v = elemPreMul<DT>(v, scaleBits);
+        if (pre) v = elemPreMul<DT>(v, scale[j]);
         acc = elemOp<DT, OP>(acc, v);
       }
     if (post) acc = elemPostDiv<DT>(acc, divisor);
@@ -740,6 +845,49 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
       if (j < nd) storeElem<ES>((char*)dst[j] + byteOff, i, acc);
   }
 }
+
+// Which fold a sweep uses, as one number: the plain folds by (element type, operator, sources held in registers: 2, 4
+// or 8), then the scaled sums by (element type, sources), then the plain copy.
+constexpr int kFoldScaledBase = 10 * 4 * 3;
+constexpr int kFoldCopy = kFoldScaledBase + 10 * 3;
+__device__ __forceinline__ int foldVariant(const SweepGeom& g) {
+  if (g.n <= 1) return kFoldCopy;  // plain copy, whatever the type
+  const int held = g.n <= 2 ? 0 : (g.n <= 4 ? 1 : 2);
+  if (g.scaleKind != kScaleNone) return kFoldScaledBase + g.dtype * 3 + held;  // ncclAvg / PreMulSum: a sum with a scale
+  return (g.dtype * 4 + g.op) * 3 + held;
+}
+
+#define DFCCL_FOLD_ARGS g.src, g.dst, g.n, g.nd, byteOff, nbytes, tid, nthr, g.scaleKind, scaleV, g.scaleBits
+#define DFCCL_FOLD_CASES_HELD(BASE, DT, OP, SC)                            \
+  case (BASE) + 0: foldTile<DT, OP, 2, SC>(DFCCL_FOLD_ARGS); break;        \
+  case (BASE) + 1: foldTile<DT, OP, 4, SC>(DFCCL_FOLD_ARGS); break;        \
+  case (BASE) + 2: foldTile<DT, OP, 8, SC>(DFCCL_FOLD_ARGS); break;
+#define DFCCL_FOLD_CASES_TYPE(DT)                                          \
+  DFCCL_FOLD_CASES_HELD((DT * 4 + kSum) * 3, DT, kSum, false)              \
+  DFCCL_FOLD_CASES_HELD((DT * 4 + kProd) * 3, DT, kProd, false)            \
+  DFCCL_FOLD_CASES_HELD((DT * 4 + kMax) * 3, DT, kMax, false)              \
+  DFCCL_FOLD_CASES_HELD((DT * 4 + kMin) * 3, DT, kMin, false)              \
+  DFCCL_FOLD_CASES_HELD(kFoldScaledBase + DT * 3, DT, kSum, true)
+__device__ __forceinline__ void foldTileAny(int variant, const SweepGeom& g, uint64_t scaleV, int64_t byteOff,
+                                            size_t nbytes, int tid, int nthr) {
+  static_assert(kI8 == 0 && kBF16 == 9, "the variants are numbered by the element types 0..9");
+  switch (variant) {
+    DFCCL_FOLD_CASES_TYPE(kI8)
+    DFCCL_FOLD_CASES_TYPE(kU8)
+    DFCCL_FOLD_CASES_TYPE(kI32)
+    DFCCL_FOLD_CASES_TYPE(kU32)
+    DFCCL_FOLD_CASES_TYPE(kI64)
+    DFCCL_FOLD_CASES_TYPE(kU64)
+    DFCCL_FOLD_CASES_TYPE(kF16)
+    DFCCL_FOLD_CASES_TYPE(kF32)
+    DFCCL_FOLD_CASES_TYPE(kF64)
+    DFCCL_FOLD_CASES_TYPE(kBF16)
+    default: foldTile<kI8, kSum, 1, false>(DFCCL_FOLD_ARGS); break;
+  }
+}
+#undef DFCCL_FOLD_CASES_TYPE
+#undef DFCCL_FOLD_CASES_HELD
+#undef DFCCL_FOLD_ARGS
 
 // The sweep of the direct protocol.  A tile is my rank's chunk in one channel slot of one loop: tile t lies in
 // loop t / C, slot t % C, at l * loop + (slot * tn + tme) * real (tn = ranks that share the index space, tme = my
@@ -753,9 +901,11 @@ __device__ __forceinline__ void foldTile(const uint64_t (&src)[kMaxDirectRanks],
 //    decides when the collective is done.  The next tile is requested while the current one is folded.  Every
 //    workgroup draws exactly one number past the end per instance, so the counter advances by exactly T.
 // At most maxTiles tiles are processed; `finished` says that no tile is left.
-template <int DT, int OP, int NS, bool SC = false>
-__device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, int64_t& posInOut, int64_t maxTiles,
-                                           int tid, int nthr, int64_t& tilesDone, bool& finished) {
+// `variant` (foldVariant) picks the fold for the element type, the operator and the number of sources; it is
+// looked up once per tile (one indexed branch), so that the loop around it exists once and not once per variant.
+__device__ __forceinline__ void sweepTiles(const SweepGeom& g, int variant, uint64_t scaleV, uint64_t* slots,
+                                           int64_t& posInOut, int64_t maxTiles, int tid, int nthr, int64_t& tilesDone,
+                                           bool& finished) {
   const bool dynamic = g.C > 1;
   DFCCL_GLOBAL uint64_t* ctr = (DFCCL_GLOBAL uint64_t*)(uintptr_t)g.ctr;
   int64_t pos = posInOut, done = 0;
@@ -773,7 +923,7 @@ __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, 
         if (tid == 0)
           slots[par] = __hip_atomic_fetch_add(ctr, 1ull, __ATOMIC_RELAXED, DFCCL_AGENT) - g.instBase + (uint64_t)g.C;
         __syncthreads();
-        tile = slots[par];
+        tile = DFCCL_UNIFORM(slots[par]);
         par ^= 1u;
       }
     }
@@ -790,14 +940,12 @@ __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, 
     const int64_t real = ((int64_t)l == g.L - 1) ? g.lastReal : g.chunkElems;
     const int64_t off = (int64_t)l * g.loop + ((int64_t)slot * g.tn + g.tme) * real;
     const int64_t nelem = (g.count - off < real) ? g.count - off : real;
-    if (nelem > 0)
-      foldTile<DT, OP, NS, SC>(g.src, g.dst, g.n, g.nd, off * g.es, (size_t)(nelem * g.es), tid, nthr, g.scaleKind,
-                               g.scaleBits);
+    if (nelem > 0) foldTileAny(variant, g, scaleV, off * g.es, (size_t)(nelem * g.es), tid, nthr);
     done++;
     if (prefetch) {
       if (tid == 0) slots[par] = nxt;
       __syncthreads();
-      tile = slots[par];
+      tile = DFCCL_UNIFORM(slots[par]);
       par ^= 1u;
       have = true;
     }
@@ -807,42 +955,11 @@ __device__ __forceinline__ void sweepFoldN(const SweepGeom& g, uint64_t* slots, 
   finished = fin;
 }
 
-template <int DT, int OP, bool SC = false>
-__device__ __forceinline__ void sweepFold(const SweepGeom& g, uint64_t* slots, int64_t& pos, int64_t maxTiles, int tid,
-                                          int nthr, int64_t& tilesDone, bool& finished) {
-  if (g.n <= 2) {
-    sweepFoldN<DT, OP, 2, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
-  } else if (g.n <= 4) {
-    sweepFoldN<DT, OP, 4, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
-  } else {
-    sweepFoldN<DT, OP, 8, SC>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
-  }
-}
-
-template <int DT>
-__device__ __forceinline__ void sweepFoldOp(int op, const SweepGeom& g, uint64_t* slots, int64_t& pos, int64_t maxTiles,
-                                            int tid, int nthr, int64_t& tilesDone, bool& finished) {
-  switch (op) {
-    case kSum: sweepFold<DT, kSum>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
-    case kProd: sweepFold<DT, kProd>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
-    case kMax: sweepFold<DT, kMax>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
-    default: sweepFold<DT, kMin>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished); break;
-  }
-}
-
 // `tid` of `nthr` threads take part (the whole workgroup, or wave 0 alone); the geometry is the same in all of them.
-__device__ __forceinline__ void sweepFoldAny(const SweepGeom& g, uint64_t* slots, int64_t& pos, int64_t maxTiles,
-                                             int tid, int nthr, int64_t& tilesDone, bool& finished) {
-  const int op = g.op;
-  if (g.n <= 1) {  // plain copy, whatever the type
-    sweepFoldN<kI8, kSum, 1>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
-    return;
-  }
-  if (g.scaleKind != kScaleNone) {  // ncclAvg / PreMulSum: a sum with a scale
-    DFCCL_FOR_DTYPE(g.dtype, (sweepFold<DT, kSum, true>(g, slots, pos, maxTiles, tid, nthr, tilesDone, finished)));
-    return;
-  }
-  DFCCL_FOR_DTYPE(g.dtype, sweepFoldOp<DT>(op, g, slots, pos, maxTiles, tid, nthr, tilesDone, finished));
+// `scaleV`: pre-multiplied sums only; lane t of every wave holds the scalar of the rank whose input is g.src[t].
+__device__ __forceinline__ void sweepFoldAny(const SweepGeom& g, uint64_t scaleV, uint64_t* slots, int64_t& pos,
+                                             int64_t maxTiles, int tid, int nthr, int64_t& tilesDone, bool& finished) {
+  sweepTiles(g, foldVariant(g), scaleV, slots, pos, maxTiles, tid, nthr, tilesDone, finished);
 }
 
 // ------------------------------------------------------------- FIFO ring protocol
@@ -852,28 +969,57 @@ __device__ __forceinline__ void sweepFoldAny(const SweepGeom& g, uint64_t* slots
 // a barrier.  (Role of the resumable runRing bodies and genericOp; see
 // ring_schedule.h for the per-step roles.)
 __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
-  const CollPlan& P = sh.plan;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int kind = P.kind, n = P.nRanks, C = P.nChannels, es = P.elemSize;
-  const int64_t count = P.count;
+  const int lane = tid & 63, wave = DFCCL_UNIFORM(tid >> 6);
+  // the plan and the position, taken from LDS into scalar registers (see DFCCL_UNIFORM)
+  struct {
+    int kind, dtype, op, root, nRanks, rank, slicesPerChunk, fifoSlots, scaleKind;
+    int64_t chunkElems, alignElems, sliceElems, slotBytes;
+    ConnFlags *sendFlags, *recvFlags;
+  } P;
+  P.kind = DFCCL_UNIFORM(sh.plan.kind);
+  P.dtype = DFCCL_UNIFORM(sh.plan.dtype);
+  P.op = DFCCL_UNIFORM(sh.plan.op);
+  P.root = DFCCL_UNIFORM(sh.plan.root);
+  P.nRanks = DFCCL_UNIFORM(sh.plan.nRanks);
+  P.rank = DFCCL_UNIFORM(sh.plan.rank);
+  P.slicesPerChunk = DFCCL_UNIFORM(sh.plan.slicesPerChunk);
+  P.fifoSlots = DFCCL_UNIFORM(sh.plan.fifoSlots);
+  P.scaleKind = DFCCL_UNIFORM(sh.plan.scaleKind);
+  P.chunkElems = DFCCL_UNIFORM(sh.plan.chunkElems);
+  P.alignElems = DFCCL_UNIFORM(sh.plan.alignElems);
+  P.sliceElems = DFCCL_UNIFORM(sh.plan.sliceElems);
+  P.slotBytes = DFCCL_UNIFORM(sh.plan.slotBytes);
+  P.sendFlags = DFCCL_UNIFORM(sh.plan.sendFlags);
+  P.recvFlags = DFCCL_UNIFORM(sh.plan.recvFlags);
+  const int kind = P.kind, n = P.nRanks, C = DFCCL_UNIFORM(sh.plan.nChannels), es = DFCCL_UNIFORM(sh.plan.elemSize);
+  const int64_t count = DFCCL_UNIFORM(sh.plan.count);
   const int64_t loop = loopElems(kind, n, C, P.chunkElems);
   const int nsteps = stepsPerLoop(kind, n);
-  const char* sendbuff = (const char*)sh.dyn.sendbuff;
-  char* recvbuff = (char*)sh.dyn.recvbuff;
-  char* sendFifo = P.sendFifo + (int64_t)ch * P.fifoChanStride;
-  const char* recvFifo = P.recvFifo + (int64_t)ch * P.fifoChanStride;
+  const char* sendbuff = (const char*)DFCCL_UNIFORM(sh.dyn.sendbuff);
+  char* recvbuff = (char*)DFCCL_UNIFORM(sh.dyn.recvbuff);
+  const int64_t fifoChanStride = DFCCL_UNIFORM(sh.plan.fifoChanStride);
+  char* sendFifo = DFCCL_UNIFORM(sh.plan.sendFifo) + (int64_t)ch * fifoChanStride;
+  const char* recvFifo = DFCCL_UNIFORM(sh.plan.recvFifo) + (int64_t)ch * fifoChanStride;
   int inPlace;
   if (kind == kAllGather) {
     inPlace = (sendbuff == recvbuff + (int64_t)P.rank * count * es);
   } else {
     inPlace = (sendbuff == recvbuff);
   }
+  // this rank's scalar of a scaled sum: from the plan, or read from device memory at every visit of an instance
+  // (a value that changes while the instance runs is the caller's affair, as in the reference)
+  uint64_t scaleBits = DFCCL_UNIFORM(sh.plan.scaleBits);
+  if (P.scaleKind == kScalePre) {
+    const void* scalePtr = DFCCL_UNIFORM(sh.plan.scalePtr);
+    if (scalePtr != nullptr) scaleBits = uniform64(loadScalar(scalePtr, es));
+    if (n == 1) inPlace = 0;  // a one-rank communicator still multiplies: its copy may not be skipped
+  }
 
-  int64_t grid = sh.dyn.gridOffset;
-  int step0 = sh.dyn.step, slice0 = sh.dyn.slice;
-  uint64_t sendStep = sh.dyn.sendStep, recvStep = sh.dyn.recvStep;
-  int64_t threshold = sh.threshold;  // the visit's spin budget (every thread keeps the same copy)
-  int64_t slicesSinceLoad = 0;       // slices this visit has moved
+  int64_t grid = DFCCL_UNIFORM(sh.dyn.gridOffset);
+  int step0 = DFCCL_UNIFORM(sh.dyn.step), slice0 = DFCCL_UNIFORM(sh.dyn.slice);
+  uint64_t sendStep = DFCCL_UNIFORM(sh.dyn.sendStep), recvStep = DFCCL_UNIFORM(sh.dyn.recvStep);
+  int64_t threshold = DFCCL_UNIFORM(sh.threshold);  // the visit's spin budget (every thread keeps the same copy)
+  int64_t slicesSinceLoad = 0;                      // slices this visit has moved over a link
 
   for (; grid < count; grid += loop, step0 = 0) {
     const int64_t real = realChunkElems(kind, n, C, P.chunkElems, P.alignElems, count, grid);
@@ -892,7 +1038,7 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
           bool ok = true;
           if (wave == 0) ok = waitDescs(A, sh, lane, w0, w1, d.recv != 0, threshold, slicesSinceLoad).ok;
           __syncthreads();
-          if (wave != 0) ok = sh.waitOk != 0;
+          if (wave != 0) ok = DFCCL_UNIFORM(sh.waitOk) != 0;
           if (!ok) {
             if (tid == 0) {
               sh.dyn.gridOffset = grid;
@@ -925,12 +1071,11 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
         if (s0 != nullptr && d0 != nullptr) {
           // a scaled sum (ncclAvg / PreMulSum) multiplies the user's input where it enters (source 0 of a step that
           // reads it) and divides where the final value is produced
-          const bool scaledStep = P.scaleKind != kScaleNone && n > 1 &&
-                                  ((P.scaleKind == kScalePre && d.useIn) || (P.scaleKind == kScalePost && d.post));
+          const bool scaledStep = (P.scaleKind == kScalePre && d.useIn) || (P.scaleKind == kScalePost && d.post);
           if (scaledStep) {
             ScaleUse su;
             su.scale.kind = P.scaleKind;
-            su.scale.bits = P.scaleBits;
+            su.scale.bits = scaleBits;
             su.preMask = d.useIn ? 1u : 0u;
             su.post = d.post != 0;
             moveSliceScaled(P.dtype, s0, s1, d0, d1, (size_t)(len * es), tid, su);
@@ -958,7 +1103,10 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
       }
     }
   }
-  if (tid == 0) {
+  // (only if a slice has gone over a link: its barrier then lies between the other threads' reading of the
+  // counters at the top and this; a visit that finds nothing left to do must not write what slower threads may
+  // still be reading, even though it would write the same values)
+  if (tid == 0 && slicesSinceLoad > 0) {
     sh.dyn.sendStep = sendStep;
     sh.dyn.recvStep = recvStep;
   }
@@ -967,11 +1115,34 @@ __device__ __forceinline__ int runFifo(const DaemonArgs& A, WgShared& sh, int ch
 
 // ----------------------------------------------------------------- direct protocol
 
-// The value lane `srcLane` of the wave holds (srcLane is the same in every lane): a register read, no LDS.
-__device__ __forceinline__ uint64_t readLane64(uint64_t v, int srcLane) {
-  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, srcLane);
-  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), srcLane);
-  return (uint64_t)lo | ((uint64_t)hi << 32);
+// Every field of the sweep's geometry is the same in every thread (it was built from the plan, or copied from
+// LDS): into scalar registers with all of it.
+__device__ __forceinline__ void uniformGeom(SweepGeom& g) {
+  g.count = (int64_t)uniform64((uint64_t)g.count);
+  g.loop = (int64_t)uniform64((uint64_t)g.loop);
+  g.chunkElems = (int64_t)uniform64((uint64_t)g.chunkElems);
+  g.lastReal = (int64_t)uniform64((uint64_t)g.lastReal);
+  g.L = (int64_t)uniform64((uint64_t)g.L);
+  g.T = (int64_t)uniform64((uint64_t)g.T);
+  g.instBase = uniform64(g.instBase);
+  g.ctr = uniform64(g.ctr);
+  g.n = __builtin_amdgcn_readfirstlane(g.n);
+  g.C = __builtin_amdgcn_readfirstlane(g.C);
+  g.ch = __builtin_amdgcn_readfirstlane(g.ch);
+  g.es = __builtin_amdgcn_readfirstlane(g.es);
+  g.me = __builtin_amdgcn_readfirstlane(g.me);
+  g.dtype = __builtin_amdgcn_readfirstlane(g.dtype);
+  g.op = __builtin_amdgcn_readfirstlane(g.op);
+  g.nd = __builtin_amdgcn_readfirstlane(g.nd);
+  g.tn = __builtin_amdgcn_readfirstlane(g.tn);
+  g.tme = __builtin_amdgcn_readfirstlane(g.tme);
+  g.scaleKind = __builtin_amdgcn_readfirstlane(g.scaleKind);
+  g.scaleBits = uniform64(g.scaleBits);
+#pragma unroll
+  for (int t = 0; t < kMaxDirectRanks; t++) {
+    g.src[t] = uniform64(g.src[t]);
+    g.dst[t] = uniform64(g.dst[t]);
+  }
 }
 
 // Wave 0, after the wait for the peers' publications: lanes 0..n-1 hold the peers' send words, lanes
@@ -1014,7 +1185,7 @@ __device__ __forceinline__ void layOutSweep(SweepGeom& g, const CollPlan& P, int
   g.me = me;
   g.dtype = P.dtype;
   g.op = P.op;
-  g.scaleKind = (folds && n > 1) ? P.scaleKind : (int)kScaleNone;
+  g.scaleKind = folds ? P.scaleKind : (int)kScaleNone;
   g.scaleBits = P.scaleBits;
   g.pad1 = 0;
 }
@@ -1042,7 +1213,7 @@ __device__ __forceinline__ void layOutSweep(SweepGeom& g, const CollPlan& P, int
 // the FIFO ring's staging of every slice through HBM at every step.
 // Two waits per instance whatever its size; each is a WaitDesc and can preempt.
 // dyn.step is the phase (0 = sweep, 2 = only the final wait is left),
-// dyn.gridOffset the sweep's position (see sweepFoldN), dyn.slice whether the
+// dyn.gridOffset the sweep's position (see sweepTiles), dyn.slice whether the
 // instance is published.
 //
 // Small collectives (the low-latency path): when the whole share of this rank is one tile of at most
@@ -1050,33 +1221,34 @@ __device__ __forceinline__ void layOutSweep(SweepGeom& g, const CollPlan& P, int
 // other inside one wave, with every decision in registers and not one workgroup barrier in between, while the
 // other waves go straight to the barrier that ends the visit.  The steps, the memory ordering and the saved
 // state are the same as for the whole workgroup; only who takes part differs.
-__device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
+// `solo`: the collective was marked at launch as one that wave 0 runs alone (soloCollective); only wave 0 is here then.
+__device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int ch, int tid, const bool solo) {
   const CollPlan& P = sh.plan;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int n = P.nRanks, C = P.nChannels, me = P.rank;
-  const int64_t L = P.loopsPerInstance;
+  const int lane = tid & 63, wave = DFCCL_UNIFORM(tid >> 6);
+  const int n = DFCCL_UNIFORM(P.nRanks), C = DFCCL_UNIFORM(P.nChannels), me = DFCCL_UNIFORM(P.rank);
+  const int64_t L = DFCCL_UNIFORM(P.loopsPerInstance);
   const int64_t forceEvery = A.knobs.forceQuitEvery;
-  const bool solo = C == 1 && L == 1 && forceEvery == 0 && P.lastChunkElems * P.elemSize <= kSoloMaxBytes;
-  // (the plan does not change during a visit, so every wave decides alike; what the other waves return is not
-  // looked at: thread 0 reports the outcome)
-  if (solo && wave != 0) return kRunDone;
-  const int nthr = solo ? 64 : kWgThreads;   // threads that take part from here on
+  const int nthr = solo ? 64 : kWgThreads;   // threads that take part
   const int mtid = solo ? lane : tid;
 
-  const uint64_t inst = sh.dyn.instance;
+  const uint64_t inst = DFCCL_UNIFORM(sh.dyn.instance);
   const uint64_t base = inst * (uint64_t)L;
-  const uint64_t sendbuff = sh.dyn.sendbuff, recvbuff = sh.dyn.recvbuff;
-  const int published = sh.dyn.slice;
-  const int peersLoaded = solo ? 0 : sh.peersLoaded;  // (a wave on its own keeps the sweep's geometry in registers)
+  const uint64_t sendbuff = DFCCL_UNIFORM(sh.dyn.sendbuff), recvbuff = DFCCL_UNIFORM(sh.dyn.recvbuff);
+  const int published = DFCCL_UNIFORM(sh.dyn.slice);
+  // (a wave on its own keeps the sweep's geometry in registers)
+  const int peersLoaded = solo ? 0 : DFCCL_UNIFORM(sh.peersLoaded);
   const int pubStride = C * (int)sizeof(PeerPub), ctrStride = C * 8;
-  PeerPub* myPub = &P.pubs[(size_t)me * C + ch];
-  const int64_t l0 = sh.dyn.gridOffset;
-  const int phase = sh.dyn.step;
-  int64_t threshold = sh.threshold;  // the visit's spin budget (every thread keeps the same copy)
-  int64_t slicesSinceLoad = 0;       // tiles this visit has moved
+  PeerPub* const pubs = DFCCL_UNIFORM(P.pubs);
+  uint64_t* const p1 = DFCCL_UNIFORM(P.p1);
+  const int scaleKind = DFCCL_UNIFORM(P.scaleKind);
+  PeerPub* myPub = &pubs[(size_t)me * C + ch];
+  const int64_t l0 = DFCCL_UNIFORM(sh.dyn.gridOffset);
+  const int phase = DFCCL_UNIFORM(sh.dyn.step);
+  int64_t threshold = DFCCL_UNIFORM(sh.threshold);  // the visit's spin budget (every thread keeps the same copy)
+  int64_t slicesSinceLoad = 0;                      // tiles this visit has moved
   // With other collectives queued a wait is only a look: switching is cheap here (contexts are small and
   // nothing is held while parked), and the workgroup is better off moving the next collective's data.
-  const int64_t cap = (sh.numActive > 1 && forceEvery == 0) ? kSoftWaitSpins : 0;
+  const int64_t cap = (DFCCL_UNIFORM(sh.numActive) > 1 && forceEvery == 0) ? kSoftWaitSpins : 0;
   // every thread has taken its copy of the position before thread 0 changes it
   if (solo) {
     DFCCL_WAVE_LDS_SYNC();
@@ -1084,26 +1256,35 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
     __syncthreads();
   }
 
-  if (!published && tid < 2) {
-    // the words carry their own instance tag: no ordering between them is needed, and the buffers' contents
-    // were made visible by whoever wrote them before the submission
-    const uint64_t tag = pubTag(inst);
-    __hip_atomic_store(G(tid == 0 ? &myPub->send : &myPub->recv), (tid == 0 ? sendbuff : recvbuff) | tag,
-                       __ATOMIC_RELAXED, DFCCL_AGENT);
-    if (tid == 0) sh.dyn.slice = 1;
+  if (!published && tid == 0) {
+    publishBuffers(myPub, sendbuff, recvbuff, inst, sh.plan.scalePtr, sh.plan.elemSize);
+    sh.dyn.slice = 1;
   }
 
   if (phase == 0) {
     SweepGeom g;
+    uint64_t scaleV = 0;  // pre-multiplied sums: lane t holds the scalar of the rank whose input is source t of the fold
     if (!peersLoaded) {
       bool ok = true;
       if (wave == 0) {
         // lanes 0..n-1 watch the peers' send words, lanes 32..32+n-1 their receive words
-        const WaitDesc w0 = waitFor(&P.pubs[ch].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
-        const WaitDesc w1 = waitFor(&P.pubs[ch].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
+        const WaitDesc w0 = waitFor(&pubs[ch].send, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
+        const WaitDesc w1 = waitFor(&pubs[ch].recv, pubTag(inst) >> 48, pubStride, n | kWaitTagged);
         const WaitResult r = waitDescs(A, sh, lane, w0, w1, true, threshold, slicesSinceLoad, cap);
         ok = r.ok;
         if (ok) {
+          // a pre-multiplied sum scales every rank's input by that rank's own scalar, found next to its
+          // pointers (written before them: the wait's acquire has made it visible)
+          if (scaleKind == kScalePre) {
+            uint64_t scaleWord = 0;
+            if (lane < n) scaleWord = __hip_atomic_load(G(&pubs[(size_t)lane * C + ch].scale), __ATOMIC_RELAXED, DFCCL_AGENT);
+            // source t of the fold is rank first + t (layOutSweep)
+            int sr = ((P.kind == kReduce) ? P.root : me) + 1 + (lane & (kMaxDirectRanks - 1));
+            if (sr >= n) sr -= n;
+            if (sr >= n) sr = 0;
+            scaleV = __shfl(scaleWord, sr);
+            if (!solo && lane < kMaxDirectRanks) sh.sweepScale[lane] = scaleV;
+          }
           layOutSweep(g, P, ch, inst, r.word);
           if (tid == 0) trace(A, sh, kTrLaidOut, 0);
           if (!solo && lane == 0) {
@@ -1114,16 +1295,15 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
       }
       if (!solo) {
         __syncthreads();
-        if (wave != 0) ok = sh.waitOk != 0;
+        if (wave != 0) ok = DFCCL_UNIFORM(sh.waitOk) != 0;
       }
       if (!ok) return kRunPreempted;  // position unchanged
     }
-    if (!solo) g = sh.sweep;
-#pragma unroll
-    for (int t = 0; t < kMaxDirectRanks; t++) {
-      g.src[t] = uniform64(g.src[t]);
-      g.dst[t] = uniform64(g.dst[t]);
+    if (!solo) {
+      g = sh.sweep;
+      if (scaleKind == kScalePre) scaleV = sh.sweepScale[lane & (kMaxDirectRanks - 1)];
     }
+    uniformGeom(g);
 
     if (tid == 0) trace(A, sh, kTrMoveBegin, 0);
     int64_t pos = l0, tilesDone = 0;
@@ -1142,7 +1322,7 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
           }
           return kRunPreempted;
         }
-        sweepFoldAny(g, sh.ticket, pos, 1, mtid, nthr, tilesDone, finished);
+        sweepFoldAny(g, scaleV, sh.ticket, pos, 1, mtid, nthr, tilesDone, finished);
         slicesSinceLoad += tilesDone;
         if (tid == 0 && tilesDone > 0) {
           sh.progressed = 1;
@@ -1150,7 +1330,7 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
         }
       }
     } else {
-      sweepFoldAny(g, sh.ticket, pos, INT64_MAX, mtid, nthr, tilesDone, finished);
+      sweepFoldAny(g, scaleV, sh.ticket, pos, INT64_MAX, mtid, nthr, tilesDone, finished);
       if (tid == 0) {
         trace(A, sh, kTrFolded, 0);
         sh.progressed = 1;
@@ -1169,7 +1349,7 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
       trace(A, sh, kTrMoveEnd, 0);
       if (!solo) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
       sh.released = 1;
-      __hip_atomic_store(G(&P.p1[(size_t)me * C + ch]), base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
+      __hip_atomic_store(G(&p1[(size_t)me * C + ch]), base + (uint64_t)L, __ATOMIC_RELAXED, DFCCL_AGENT);
       trace(A, sh, kTrPosted, 1);
     }
   }
@@ -1177,12 +1357,12 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
   // every chunk of my receive buffer is written, and nobody reads my send buffer any more
   if (phase != 0 && tid == 0) sh.released = 1;  // resumed here: the sweep's release was done before it was parked
   {
-    const WaitDesc w0 = waitFor(&P.p1[ch], base + (uint64_t)L, ctrStride, n);
+    const WaitDesc w0 = waitFor(&p1[ch], base + (uint64_t)L, ctrStride, n);
     bool ok = true;
     if (wave == 0) ok = waitDescs(A, sh, lane, w0, noWait(), true, threshold, slicesSinceLoad, cap).ok;
     if (!solo) {
       __syncthreads();
-      if (wave != 0) ok = sh.waitOk != 0;
+      if (wave != 0) ok = DFCCL_UNIFORM(sh.waitOk) != 0;
     }
     if (!ok) {
       if (tid == 0) {
@@ -1199,9 +1379,16 @@ __device__ __forceinline__ int runDirect(const DaemonArgs& A, WgShared& sh, int 
   return kRunDone;
 }
 
-__device__ __forceinline__ int runColl(const DaemonArgs& A, WgShared& sh, int ch, int tid) {
-  if (sh.plan.proto == kProtoDirect) return runDirect(A, sh, ch, tid);
+__device__ __forceinline__ int runColl(const DaemonArgs& A, WgShared& sh, int ch, int tid, const bool solo) {
+  if (solo || DFCCL_UNIFORM(sh.plan.proto) == kProtoDirect) return runDirect(A, sh, ch, tid, solo);
   return runFifo(A, sh, ch, tid);
+}
+
+// Whether wave 0 runs a collective alone (decided once per launch, from the plan): a direct collective whose whole
+// share of this rank is one tile of at most kSoloMaxBytes, and no forced preemption points asked for.
+__device__ __forceinline__ bool soloCollective(const DFCCL_GLOBAL CollPlan* pl, int64_t forceQuitEvery) {
+  return pl->proto == kProtoDirect && pl->nChannels == 1 && pl->loopsPerInstance == 1 && forceQuitEvery == 0 &&
+         pl->lastChunkElems * pl->elemSize <= kSoloMaxBytes;
 }
 
 // One thread: the resident collective has finished an instance.  Resets its position for the next instance
@@ -1244,57 +1431,92 @@ __device__ __forceinline__ void completeColl(const DaemonArgs& A, const RankDev&
   storeStruct(&R.dyn[(size_t)ch * R.nColls + coll], sh.dyn);
 }
 
-// Visit one collective of the task queue: make its context resident, run it,
-// then post the completion or save the context.
-__device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int tid, int qi) {
+// One thread, at the start of a visit: make the collective's context resident and set the visit's spin budget.
+__device__ __forceinline__ void beginVisit(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, uint32_t coll,
+                                           int qi) {
   const Knobs& K = A.knobs;
-  const uint32_t coll = sh.taskq[qi];
-  DynCtx* dynG = &R.dyn[(size_t)ch * R.nColls + coll];
-  if (tid == 0) {
-    if (sh.loadedColl != (int32_t)coll) {
-      loadStruct(sh.plan, &R.plans[coll]);
-      loadStruct(sh.dyn, dynG);
-      sh.loadedColl = (int32_t)coll;
-      sh.peersLoaded = 0;
-      sh.stats.ctxLoads++;
-    }
-    sh.dyn.tryCnt++;
-    // spin budget of this visit: BASE * min(tries, NUM_TRY); the queue head is given NUM_TRY times more
-    const int64_t tries = sh.dyn.tryCnt < K.numTryTaskqHead ? sh.dyn.tryCnt : K.numTryTaskqHead;
-    int64_t thr = K.baseCtxSwitchThreshold * tries;
-    if (qi == 0) thr *= K.numTryTaskqHead;
-    sh.threshold = thr < 1 ? 1 : thr;
-    sh.waitOk = 1;
-    sh.progressed = 0;
-    sh.released = 0;
-    sh.dyn.wait[0] = noWait();
-    sh.dyn.wait[1] = noWait();
-    trace(A, sh, kTrVisitBegin, coll);
+  if (sh.loadedColl != (int32_t)coll) {
+    loadStruct(sh.plan, &R.plans[coll]);
+    loadStruct(sh.dyn, &R.dyn[(size_t)ch * R.nColls + coll]);
+    sh.loadedColl = (int32_t)coll;
+    sh.peersLoaded = 0;
+    sh.stats.ctxLoads++;
   }
-  __syncthreads();
-  if (tid == 0) trace(A, sh, kTrRunEntry, 0);
-  const int status = runColl(A, sh, ch, tid);
-  if (tid == 0) trace(A, sh, kTrRunReturned, (uint32_t)status);
-  __syncthreads();
-  if (tid == 0) {
-    if (sh.progressed) sh.progressedRound = 1;
-    if (status == kRunDone) {
-      sh.taskq[qi] = (uint16_t)kInvalidTask;
-      completeColl(A, R, sh, ch, coll);
-    } else {
-      // preempted: save the context (saveExcutingCollCtx, enqueue_ofccl_dev.cu:664-677)
-      storeStruct(dynG, sh.dyn);
-      sh.stats.ctxSaves++;
-    }
-    trace(A, sh, kTrVisitEnd, (uint32_t)status);
-  }
-  __syncthreads();
+  sh.dyn.tryCnt++;
+  // spin budget of this visit: BASE * min(tries, NUM_TRY); the queue head is given NUM_TRY times more
+  const int64_t tries = sh.dyn.tryCnt < K.numTryTaskqHead ? sh.dyn.tryCnt : K.numTryTaskqHead;
+  int64_t thr = K.baseCtxSwitchThreshold * tries;
+  if (qi == 0) thr *= K.numTryTaskqHead;
+  sh.threshold = thr < 1 ? 1 : thr;
+  sh.waitOk = 1;
+  sh.progressed = 0;
+  sh.released = 0;
+  sh.dyn.wait[0] = noWait();
+  sh.dyn.wait[1] = noWait();
+  trace(A, sh, kTrVisitBegin, coll);
 }
 
-extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const DaemonArgs* __restrict__ argsPtr) {
+// One thread, at the end of a visit: post the completion, or save the context.
+__device__ __forceinline__ void endVisit(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, uint32_t coll, int qi,
+                                         int status) {
+  if (sh.progressed) sh.progressedRound = 1;
+  if (status == kRunDone) {
+    sh.taskq[qi] = (uint16_t)kInvalidTask;
+    completeColl(A, R, sh, ch, coll);
+  } else {
+    // preempted: save the context (saveExcutingCollCtx, enqueue_ofccl_dev.cu:664-677)
+    storeStruct(&R.dyn[(size_t)ch * R.nColls + coll], sh.dyn);
+    sh.stats.ctxSaves++;
+  }
+  trace(A, sh, kTrVisitEnd, (uint32_t)status);
+}
+
+// Visit one collective of the task queue: make its context resident, run it,
+// then post the completion or save the context.
+// `solo` (from the round's readySolo bitmap, the same in every thread): wave 0 does all of that by itself, its
+// lane 0 in the part of thread 0, without a workgroup barrier from the context to the completion entry; the
+// other waves touch nothing and wait at the barrier that ends the visit.
+__device__ __forceinline__ void visit(const DaemonArgs& A, const RankDev& R, WgShared& sh, int ch, int tid, int wave, int qi,
+                                      const bool solo) {
+  const int lane = tid & 63;
+  const bool first = solo ? (wave == 0 && lane == 0) : (tid == 0);  // the thread that does the bookkeeping
+  uint32_t coll = 0;
+  if (solo) {
+    if (wave == 0) {
+      if (first) {
+        coll = sh.taskq[qi];
+        beginVisit(A, R, sh, ch, coll, qi);
+      }
+      DFCCL_WAVE_LDS_SYNC();  // (the context lane 0 has put into LDS is what the other lanes read next)
+    }
+  } else {
+    coll = DFCCL_UNIFORM((uint32_t)sh.taskq[qi]);
+    if (first) beginVisit(A, R, sh, ch, coll, qi);
+    __syncthreads();
+  }
+  int status = kRunDone;
+  if (!solo || wave == 0) {  // (one call for both cases: the movers are inlined into it)
+    if (first) trace(A, sh, kTrRunEntry, 0);
+    status = runColl(A, sh, ch, tid, solo);
+    if (first) trace(A, sh, kTrRunReturned, (uint32_t)status);
+  }
+  if (solo) {
+    if (wave == 0) {
+      DFCCL_WAVE_LDS_SYNC();
+      if (first) endVisit(A, R, sh, ch, coll, qi, status);
+    }
+    __syncthreads();
+  } else {
+    __syncthreads();
+    if (first) endVisit(A, R, sh, ch, coll, qi, status);
+    __syncthreads();
+  }
+}
+
+extern "C" __global__ __launch_bounds__(kWgThreads) void DFCCL_DAEMON_KERNEL(const DaemonArgs* __restrict__ argsPtr) {
   DFCCL_WG_SHARED(WgShared, sh);
   const DaemonArgs& A = *argsPtr;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid0 = threadIdx.x, wave = DFCCL_UNIFORM(tid0 >> 6);
   // Workgroups go to the XCDs round robin.  The channels of a rank are rotated by its slot, so that the
   // leaders (channel 0), which talk to the host, do not all sit on one XCD.
   const int slot = (int)blockIdx.x / A.channelsPerRank;
@@ -1307,24 +1529,28 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
 
   // ---- restore the state a previous launch saved (blockInit, enqueue_ofccl_dev.cu:203-479)
   DFCCL_GLOBAL WgSaved& S = *G(&R.saved[ch]);
-  if (tid == 0) {
-    sh.frontier = S.frontier;
-    sh.hostFrontier = S.hostFrontier;
-    sh.publishedHead = ~0ull;
+  Wave0Regs st;  // (see Wave0Regs: only wave 0's copy is ever used)
+  st.frontier = DFCCL_WAVE_UNIFORM(S.frontier);
+  st.hostFrontier = DFCCL_WAVE_UNIFORM(S.hostFrontier);
+  st.publishedHead = ~0ull;
+  st.idle = 0;
+  st.round = 0;
+  st.statsReqSeen = 0;
+  st.numActive = 0;
+  st.ingested = 0;
+  st.allFresh = 0;
+  st.rankBusy = 0;
+  st.finalQuit = 0;
+  st.numReady = 0;
+  if (tid0 == 0) {
     sh.numActive = S.numActive;
     sh.numReady = 0;
-    sh.finalQuit = 0;
     sh.exitKind = kExitNone;
-    sh.idle = 0;
-    sh.ingested = 0;
     sh.progressedRound = 0;
     sh.loadedColl = -1;
     sh.peersLoaded = 0;
     sh.wgIndex = (uint32_t)(slot * A.channelsPerRank + ch);
     sh.traceCount = 0;
-    sh.round = 0;
-    sh.allFresh = 0;
-    sh.rankBusy = 0;
     sh.cqNext = S.cqNext;
     trace(A, sh, kTrLaunch, A.epoch);
     const DFCCL_GLOBAL WgStats* hs = G(&R.stats[ch]);
@@ -1337,89 +1563,104 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     sh.stats.slicesMoved = hs->slicesMoved;
     sh.stats.spins = hs->spins;
     sh.statsEpoch = 0;
-    sh.statsReqSeen = 0;
   }
   __syncthreads();
-  for (int i = tid; i < sh.numActive; i += kWgThreads) sh.taskq[i] = S.taskq[i];
-  for (int i = tid; i < R.nColls; i += kWgThreads) sh.collChannels[i] = (uint8_t)G(&R.plans[i])->nChannels;
+  for (int i = tid0; i < sh.numActive; i += kWgThreads) sh.taskq[i] = S.taskq[i];
+  for (int i = tid0; i < R.nColls; i += kWgThreads) {
+    const DFCCL_GLOBAL CollPlan* pl = G(&R.plans[i]);
+    sh.collChannels[i] = (uint8_t)((uint8_t)pl->nChannels | (soloCollective(pl, K.forceQuitEvery) ? kCollSolo : (uint8_t)0));
+  }
   __syncthreads();
 
   for (;;) {
-    // ---- ingest phase (wave 0)
+    // (this round's copy of the thread number: see DFCCL_FRESH_PER_ROUND)
+    int tid = tid0;
+    DFCCL_FRESH_PER_ROUND(tid);
+    const int lane = tid & 63;
+    // ---- ingest phase (wave 0; the scheduler's own state is in `st`, the same in every lane)
     if (wave == 0) {
+      st.numActive = DFCCL_WAVE_UNIFORM(sh.numActive);  // (thread 0 compacts the queue at the end of a run phase)
       if (ch == 0) {
-        pollHost(A, R, sh, lane);
+        pollHost(A, R, sh, st, lane);
       } else {
-        ingestMirror(A, R, sh, ch, lane);
+        ingestMirror(A, R, sh, st, ch, lane);
       }
-      if (DFCCL_WAVE_UNIFORM(sh.numActive) > 0) {
-        scanReady(R, sh, ch, lane);
-      } else if (lane == 0) {
-        sh.numReady = 0;
-      }
-      if (lane == 0 && sh.ingested > 0) {
+      scanReady(R, sh, st, ch, lane);
+      if (lane == 0 && st.ingested > 0) {
         trace(A, sh, kTrScanDone, 0);
       }
-      DFCCL_WAVE_LDS_SYNC();
-      if (lane == 0) {
-        // the host's requests and the lifetime limit are looked at every 8th round, and only every 64th while
-        // submissions keep arriving: nobody waits on them, and a new submission does not wait for them either
-        uint32_t abortFlag = 0, quitFlag = 0;
-        bool expired = false;
-        const uint32_t round = sh.round++;
-        if ((round & 7u) == 0 && (sh.ingested == 0 || (round & 63u) == 0)) {
-          abortFlag = __hip_atomic_load(G(&A.devFlags[1]), __ATOMIC_RELAXED, DFCCL_AGENT);
-          quitFlag = __hip_atomic_load(G(&A.devFlags[0]), __ATOMIC_RELAXED, DFCCL_AGENT);
-          const uint32_t statsReq = __hip_atomic_load(G(&A.devFlags[2]), __ATOMIC_RELAXED, DFCCL_AGENT);
-          if (statsReq != sh.statsEpoch) {
-            // the host wants the counters
-            sh.statsEpoch = statsReq;
-            flushStats(R, sh, ch, statsReq);
-          }
-          // (not in the first round of a launch: a lifetime shorter than the start-up would otherwise end every
-          // launch before its first visit, and nothing would ever move)
-          expired = K.maxLifetimeTicks > 0 && round != 0 && (int64_t)(wall_clock64() - startTick) > K.maxLifetimeTicks;
+      // The round's decisions.  The host's requests and the lifetime limit are looked at every 8th round, and only
+      // every 64th while submissions keep arriving: nobody waits on them, and a new submission does not wait for
+      // them either.
+      uint32_t abortFlag = 0, quitFlag = 0, expired = 0;
+      const uint32_t round = st.round++;
+      if ((round & 7u) == 0 && (st.ingested == 0 || (round & 63u) == 0)) {
+        abortFlag = DFCCL_WAVE_UNIFORM(__hip_atomic_load(G(&A.devFlags[1]), __ATOMIC_RELAXED, DFCCL_AGENT));
+        quitFlag = DFCCL_WAVE_UNIFORM(__hip_atomic_load(G(&A.devFlags[0]), __ATOMIC_RELAXED, DFCCL_AGENT));
+        const uint32_t statsReq = DFCCL_WAVE_UNIFORM(__hip_atomic_load(G(&A.devFlags[2]), __ATOMIC_RELAXED, DFCCL_AGENT));
+        if (lane == 0 && statsReq != sh.statsEpoch) {
+          // the host wants the counters
+          sh.statsEpoch = statsReq;
+          flushStats(R, sh, ch, statsReq);
         }
-        if (sh.ingested > 0 || sh.progressedRound) {
-          sh.idle = 0;
-        } else {
-          sh.idle++;
-        }
-        if (sh.numActive > 0 && sh.idle > 0 && (sh.idle & (kStuckReportRounds - 1)) == 0) reportStuck(R, sh, ch);
-        if (abortFlag) {
-          sh.exitKind = kExitAbort;
-        } else if (sh.finalQuit) {
-          sh.exitKind = kExitFinal;
-        } else if (quitFlag || expired) {
-          sh.exitKind = kExitVoluntary;
-        } else if (sh.idle >= K.tolerantUnprogressedCnt) {
-          // Idle for long: leave, and take the whole daemon along (every workgroup saves its state and leaves at
-          // its next look at this flag).  The kernel can only be launched again once all of it has ended, and a
-          // submission for a rank whose workgroups have left is not seen by anybody until then: a daemon that
-          // stays half resident because other ranks are busy would starve that rank.
-          sh.exitKind = kExitVoluntary;
-          __hip_atomic_store(G(&A.devFlags[0]), 1u, __ATOMIC_RELAXED, DFCCL_AGENT);
-        }
-        if (DFCCL_TEST_NEVER_LEAVES()) sh.exitKind = kExitNone;
-        sh.progressedRound = 0;
+        // (not in the first round of a launch: a lifetime shorter than the start-up would otherwise end every
+        // launch before its first visit, and nothing would ever move)
+        expired = DFCCL_WAVE_UNIFORM((uint32_t)(K.maxLifetimeTicks > 0 && round != 0 &&
+                                                (int64_t)(wall_clock64() - startTick) > K.maxLifetimeTicks));
       }
-      DFCCL_WAVE_LDS_SYNC();
-      if (DFCCL_WAVE_UNIFORM(sh.numReady) == 0 && DFCCL_WAVE_UNIFORM(sh.ingested) == 0) {
+      const int32_t progressedRound = DFCCL_WAVE_UNIFORM(sh.progressedRound);  // (set by thread 0 during the visits)
+      DFCCL_WAVE_LDS_SYNC();  // (every lane has read it before lane 0 clears it)
+      if (st.ingested > 0 || progressedRound) {
+        st.idle = 0;
+      } else {
+        st.idle++;
+      }
+      if (lane == 0 && st.numActive > 0 && st.idle > 0 && (st.idle & (kStuckReportRounds - 1)) == 0) {
+        reportStuck(R, sh, ch);
+      }
+      int exitKind = kExitNone;
+      bool takeDaemonAlong = false;
+      if (abortFlag) {
+        exitKind = kExitAbort;
+      } else if (st.finalQuit) {
+        exitKind = kExitFinal;
+      } else if (quitFlag || expired) {
+        exitKind = kExitVoluntary;
+      } else if (st.idle >= K.tolerantUnprogressedCnt) {
+        // Idle for long: leave, and take the whole daemon along (every workgroup saves its state and leaves at
+        // its next look at this flag).  The kernel can only be launched again once all of it has ended, and a
+        // submission for a rank whose workgroups have left is not seen by anybody until then: a daemon that
+        // stays half resident because other ranks are busy would starve that rank.
+        exitKind = kExitVoluntary;
+        takeDaemonAlong = true;
+      }
+      if (DFCCL_TEST_NEVER_LEAVES()) exitKind = kExitNone;
+      if (lane == 0) {
+        if (exitKind != kExitNone) {
+          sh.exitKind = exitKind;
+          if (takeDaemonAlong) __hip_atomic_store(G(&A.devFlags[0]), 1u, __ATOMIC_RELAXED, DFCCL_AGENT);
+        }
+        if (progressedRound) sh.progressedRound = 0;
+      }
+      if (st.numReady == 0 && st.ingested == 0) {
         // nothing can move: the leader's next poll is a PCIe round trip anyway, the others back off a little
         if (ch != 0) {
           __builtin_amdgcn_s_sleep(20);
-        } else if (sh.rankBusy) {
+        } else if (st.rankBusy) {
           __builtin_amdgcn_s_sleep(100);
         }
       }
+      // A run phase follows: the scheduler's registers wait in LDS meanwhile (a dozen values that would
+      // otherwise be live, and set aside lane by lane, across all of the data movement).
+      if (st.numReady > 0 && exitKind == kExitNone && lane == 0) sh.w0 = st;
     }
     __syncthreads();
     // Every thread takes this round's decisions into registers, and only then may wave 0 go on to the next
     // round and overwrite them (without the second barrier a wave that is late reading numReady could see the
     // next round's value, enter the run phase alone and leave the workgroup's barriers out of step for good).
-    const int roundExit = sh.exitKind;
-    const int nq = sh.numActive;
-    const int numReady = sh.numReady;
+    const int roundExit = DFCCL_UNIFORM(sh.exitKind);
+    const int nq = DFCCL_UNIFORM(sh.numActive);
+    const int numReady = DFCCL_UNIFORM(sh.numReady);
     __syncthreads();
     if (roundExit != kExitNone) break;
     if (tid == 0 && numReady > 0) trace(A, sh, kTrRoundDecided, (uint32_t)numReady);
@@ -1428,11 +1669,12 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
     // (traverseTaskQ, enqueue_ofccl_dev.cu:922-1016)
     if (numReady > 0) {
       for (int wd = 0; wd * 64 < nq; wd++) {
-        uint64_t m = sh.ready[wd];
+        uint64_t m = DFCCL_UNIFORM(sh.ready[wd]);
+        const uint64_t ms = DFCCL_UNIFORM(sh.readySolo[wd]);
         while (m) {
           const int b = (int)__builtin_ctzll(m);
           m &= m - 1;
-          visit(A, R, sh, ch, tid, wd * 64 + b);
+          visit(A, R, sh, ch, tid, wave, wd * 64 + b, ((ms >> b) & 1ull) != 0);
         }
       }
       // drop finished collectives from the task queue, keeping arrival order
@@ -1445,23 +1687,44 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
         sh.numActive = w;
       }
       __syncthreads();
+      // (the other waves' copies, which nobody uses, are given new values too, so that no wave has to keep the old
+      // ones across the run phase; they do not read LDS for it: wave 0 may write there again before they get here)
+      if (wave == 0) {
+        st.frontier = DFCCL_UNIFORM(sh.w0.frontier);
+        st.hostFrontier = DFCCL_UNIFORM(sh.w0.hostFrontier);
+        st.publishedHead = DFCCL_UNIFORM(sh.w0.publishedHead);
+        st.idle = DFCCL_UNIFORM(sh.w0.idle);
+        st.round = DFCCL_UNIFORM(sh.w0.round);
+        st.statsReqSeen = DFCCL_UNIFORM(sh.w0.statsReqSeen);
+        st.numActive = DFCCL_UNIFORM(sh.w0.numActive);
+        st.ingested = DFCCL_UNIFORM(sh.w0.ingested);
+        st.allFresh = DFCCL_UNIFORM(sh.w0.allFresh);
+        st.rankBusy = DFCCL_UNIFORM(sh.w0.rankBusy);
+        st.finalQuit = DFCCL_UNIFORM(sh.w0.finalQuit);
+        st.numReady = DFCCL_UNIFORM(sh.w0.numReady);
+      } else {
+        st.frontier = st.hostFrontier = st.publishedHead = 0;
+        st.idle = 0;
+        st.round = st.statsReqSeen = 0;
+        st.numActive = st.ingested = st.allFresh = st.rankBusy = st.finalQuit = st.numReady = 0;
+      }
     }
   }
 
   // ---- leave
-  const int exitKind = sh.exitKind;
+  const int exitKind = DFCCL_UNIFORM(sh.exitKind);
   if (exitKind == kExitVoluntary) {
-    for (int i = tid; i < sh.numActive; i += kWgThreads) S.taskq[i] = sh.taskq[i];
-    if (tid == 0) {
-      S.frontier = sh.frontier;
-      S.hostFrontier = sh.hostFrontier;
+    for (int i = tid0; i < sh.numActive; i += kWgThreads) S.taskq[i] = sh.taskq[i];
+    if (tid0 == 0) {
+      S.frontier = st.frontier;
+      S.hostFrontier = st.hostFrontier;
       S.numActive = sh.numActive;
       S.cqNext = sh.cqNext;
       sh.stats.voluntaryQuits++;
     }
   }
   __syncthreads();
-  if (tid == 0) {
+  if (tid0 == 0) {
     trace(A, sh, kTrExit, (uint32_t)exitKind);
     if (A.trace != nullptr)  // the last record slot of the workgroup holds how many records it wrote
       G(A.trace)[((size_t)sh.wgIndex * kTraceRecords + (kTraceRecords - 1)) * 2 + 1] = sh.traceCount;
@@ -1475,15 +1738,15 @@ extern "C" __global__ __launch_bounds__(kWgThreads) void dfcclDaemonKernel(const
 
 // Host-side launcher used by the runtime (kept here so that the kernel symbol
 // and its launch shape live in one translation unit).
-extern "C" hipError_t dfcclLaunchDaemon(const dfccl::DaemonArgs* devArgs, int nSlots, int channelsPerRank,
-                                        hipStream_t stream) {
+extern "C" hipError_t DFCCL_DAEMON_LAUNCH(const dfccl::DaemonArgs* devArgs, int nSlots, int channelsPerRank,
+                                          hipStream_t stream) {
   const unsigned grid = (unsigned)(nSlots * channelsPerRank);
   if (grid == 0) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(dfccl::dfcclDaemonKernel, dim3(grid), dim3(dfccl::kWgThreads), 0, stream, devArgs);
+  hipLaunchKernelGGL(dfccl::DFCCL_DAEMON_KERNEL, dim3(grid), dim3(dfccl::kWgThreads), 0, stream, devArgs);
   return hipGetLastError();
 }
 
 // Workgroups of the daemon kernel one CU keeps resident.
-extern "C" hipError_t dfcclDaemonOccupancy(int* perCu) {
-  return hipOccupancyMaxActiveBlocksPerMultiprocessor(perCu, dfccl::dfcclDaemonKernel, dfccl::kWgThreads, 0);
+extern "C" hipError_t DFCCL_DAEMON_OCCUPANCY(int* perCu) {
+  return hipOccupancyMaxActiveBlocksPerMultiprocessor(perCu, dfccl::DFCCL_DAEMON_KERNEL, dfccl::kWgThreads, 0);
 }

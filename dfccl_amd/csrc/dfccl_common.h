@@ -73,10 +73,15 @@ struct alignas(128) ConnFlags {
 // the reference's ptrExchange, src/collectives_ofccl/device/ofccl_prims_simple.h:737-869).
 // Each word carries the instance it belongs to in its top 16 bits (pubTag), so a peer that polls the word
 // gets the pointer with the same load that tells it the instance has started.
+// `scale` is the rank's own scalar of a pre-multiplied sum (ncclAvg on float types, PreMulSum): the peer that
+// folds this rank's input multiplies it by this rank's scalar, as the rank's own primitives would have.  The
+// host writes it at finalize; for a scalar that lives in device memory the workgroup reads it when it announces
+// an instance and stores it here before the tagged words (which it then stores with release semantics).
 struct alignas(32) PeerPub {
   uint64_t send;       // sendbuff | pubTag(instance)
   uint64_t recv;       // recvbuff | pubTag(instance)
-  uint64_t pad[2];
+  uint64_t scale;      // one element of the run dtype in the low bytes
+  uint64_t pad;
 };
 DFCCL_HD uint64_t pubTag(uint64_t instance) { return ((instance + 1) & 0xffffull) << 48; }
 
@@ -120,7 +125,8 @@ struct alignas(16) CollPlan {
   // direct protocol (peers read each other's buffers, no FIFO)
   int32_t proto;
   int32_t scaleKind;       // a Sum with a scale (ncclAvg, PreMulSum): kScaleNone / kScalePre / kScalePost of reduce_ops.h
-  uint64_t scaleBits;      // its scalar: one element of dtype in the low bytes, or the divisor
+  uint64_t scaleBits;      // this rank's scalar: one element of dtype in the low bytes, or the divisor
+  const void* scalePtr;    // PreMulSum with the scalar in device memory: read whenever an instance starts (else null)
   PeerPub* pubs;           // [nRanks][nChannels]
   uint64_t* p1;            // [nRanks][nChannels] loops whose own chunk is folded and stored everywhere
   int64_t loopsPerInstance;

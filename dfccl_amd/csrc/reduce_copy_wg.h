@@ -47,7 +47,8 @@ __host__ __device__ __forceinline__ ScaleUse noScale() {
 }
 
 // SC = false compiles the scaling away altogether (the plain ops' code is what it is without it).
-template <int DT, int OP, int NS, int ND, int U, bool NT, bool SC = false>
+// NT: non-temporal loads (every byte is read once); NTS: non-temporal stores, by default like the loads.
+template <int DT, int OP, int NS, int ND, int U, bool NT, bool SC = false, bool NTS = NT>
 __device__ __forceinline__ void reduceCopyWG(const void* const (&srcs)[NS], void* const (&dsts)[ND], size_t nbytes,
                                              int tid, int nthr, const ScaleUse su = noScale()) {
   constexpr int ES = typeSize(DT);
@@ -90,7 +91,7 @@ __device__ __forceinline__ void reduceCopyWG(const void* const (&srcs)[NS], void
         for (int s = 1; s < NS; s++) acc = packOp<DT, OP>(acc, v[s][u]);
         if (post) acc = packPostDiv<DT>(acc, divisor);
 #pragma unroll
-        for (int d = 0; d < ND; d++) storePack<NT>(dsts[d], base + (size_t)u * nthr, acc);
+        for (int d = 0; d < ND; d++) storePack<NTS>(dsts[d], base + (size_t)u * nthr, acc);
       }
     }
     for (size_t i = ntiles * tile + tid; i < npacks; i += nthr) {
@@ -104,7 +105,7 @@ __device__ __forceinline__ void reduceCopyWG(const void* const (&srcs)[NS], void
       }
       if (post) acc = packPostDiv<DT>(acc, divisor);
 #pragma unroll
-      for (int d = 0; d < ND; d++) storePack<NT>(dsts[d], i, acc);
+      for (int d = 0; d < ND; d++) storePack<NTS>(dsts[d], i, acc);
     }
     doneBytes = npacks << 4;
   }

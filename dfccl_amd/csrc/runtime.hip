@@ -32,9 +32,14 @@
 
 #define DFCCL_API extern "C" __attribute__((visibility("default")))
 
+// daemon.hip is compiled twice: the kernel that normally runs, and one that also writes the timeline stamps
+// (launched when DFCCL_TRACE=1)
 extern "C" hipError_t dfcclDaemonOccupancy(int* perCu);
+extern "C" hipError_t dfcclDaemonOccupancyTraced(int* perCu);
 extern "C" hipError_t dfcclLaunchDaemon(const dfccl::DaemonArgs* devArgs, int nSlots, int channelsPerRank,
                                         hipStream_t stream);
+extern "C" hipError_t dfcclLaunchDaemonTraced(const dfccl::DaemonArgs* devArgs, int nSlots, int channelsPerRank,
+                                              hipStream_t stream);
 
 namespace dfccl {
 
@@ -83,9 +88,13 @@ struct CommGroup {
   // a rank context that ran this collective has been destroyed: the counters in the group's device memory no
   // longer match a fresh context's, so the communicator cannot be registered again
   bool retired = false;
+  bool capacityUnknown = false;  // the device would not say how many workgroups it keeps resident (planGroup)
   int kind = 0, dtypeUser = 0, op = 0, root = 0;  // op: the element op the kernels apply (Sum for the scaled sums)
   int scaleKind = kScaleNone;                      // ncclAvg / PreMulSum: see Scale in reduce_ops.h
-  uint64_t scaleBits = 0;
+  // every rank's own scalar (a PreMulSum operator is made per rank, and a rank's input is multiplied by that
+  // rank's scalar): the bits of one element, or for an operator made with ncclScalarDevice the device address
+  // the scalar is read from whenever an instance starts.  Set by each rank's Prepare.
+  std::vector<uint64_t> scaleBits, scalePtr;
   size_t countUser = 0;
   // derived plan
   int dtype = 0, elemSize = 1, nChannels = 1, slicesPerChunk = 1, fifoSlots = 1;
@@ -107,8 +116,14 @@ struct ncclComm {
   dfccl::CommGroup* group;
   int rank;
   bool registered;
-  // reduction operators made by ncclRedOpCreatePreMulSum: op value - ncclNumOps -> {datatype, scalar bits}
-  std::map<int, std::pair<int, uint64_t>> userOps;
+  // reduction operators made by ncclRedOpCreatePreMulSum: op value - ncclNumOps -> the datatype and the scalar
+  // (its bits, or the device address it is to be read from)
+  struct UserOp {
+    int datatype;
+    uint64_t bits;
+    uint64_t devPtr;
+  };
+  std::map<int, UserOp> userOps;
   int nextUserOp = 0;
 };
 
@@ -241,6 +256,10 @@ struct Daemon {
     if (nSlots == 0) return false;
     // a multiple of 8 channels keeps channel c of every rank on XCD c % 8
     if (chans > 1) chans = (chans + 7) & ~7;
+    if (residentCapacity() <= 0) {
+      fprintf(stderr, "dfccl: cannot tell how many daemon workgroups device %d keeps resident\n", device);
+      return false;
+    }
     if ((long)nSlots * chans > residentCapacity()) {
       fprintf(stderr,
               "dfccl: %d rank slots x %d channels do not fit the %ld workgroups the GPU keeps resident; "
@@ -258,7 +277,8 @@ struct Daemon {
     if (hipMemcpy(devArgs, &hostArgs, sizeof(hostArgs), hipMemcpyHostToDevice) != hipSuccess) return false;
     if (hipMemset(devFlags, 0, 64) != hipSuccess) return false;
     if (hipStreamSynchronize(nullptr) != hipSuccess) return false;  // args and flags are in place before the launch
-    if (dfcclLaunchDaemon(devArgs, nSlots, chans, stream) != hipSuccess) return false;
+    if ((trace != nullptr ? dfcclLaunchDaemonTraced : dfcclLaunchDaemon)(devArgs, nSlots, chans, stream) != hipSuccess)
+      return false;
     if (hipEventRecord(doneEv, stream) != hipSuccess) return false;
     running = true;
     launches++;
@@ -454,12 +474,33 @@ static void destroyDaemon(Daemon* d) {
 // Rank contexts alive per device: the workgroups of all of them have to fit the GPU together.
 static std::atomic<int> gLiveRankCtxs[64];
 
-// Workgroups of the daemon kernel the device keeps resident at once (compute units x workgroups per unit).
+// Workgroups of the daemon kernel `device` keeps resident at once (compute units x workgroups per unit), asked of
+// the runtime once per device.  0 if the runtime cannot say: the callers then refuse to plan or to launch (a grid
+// that is not resident as a whole makes every collective park until the idle exit).
 static int deviceWorkgroupSlots(int device) {
-  int cus = 0, perCu = 0;
-  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
-  if (dfcclDaemonOccupancy(&perCu) != hipSuccess || perCu < 1) perCu = 1;
-  return cus * perCu;
+  static std::mutex mu;
+  static std::map<int, int> known;
+  std::lock_guard<std::mutex> lk(mu);
+  auto it = known.find(device);
+  if (it != known.end()) return it->second;
+  int cus = 0, perCu = 0, current = -1;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) return 0;
+  // the occupancy query answers for the current device
+  if (hipGetDevice(&current) != hipSuccess) return 0;
+  if (current != device && hipSetDevice(device) != hipSuccess) return 0;
+  hipError_t e = dfcclDaemonOccupancy(&perCu);
+  if (e == hipSuccess && envInt("DFCCL_TRACE", 0) != 0) {  // the traced kernel will run: it has to fit as well
+    int traced = 0;
+    e = dfcclDaemonOccupancyTraced(&traced);
+    perCu = std::min(perCu, traced);
+  }
+  if (current != device) (void)hipSetDevice(current);
+  if (e != hipSuccess || perCu < 1) return 0;
+  // One workgroup per compute unit is the design point, whatever the occupancy calculation would allow beyond
+  // that: the workgroups of a rank share its work tile by tile, and a second workgroup per unit only halves what
+  // each of them has in flight.  (What the calculation allows beyond one is headroom for residency.)
+  known[device] = cus;
+  return cus;
 }
 
 static void planGroup(CommGroup* g) {
@@ -489,8 +530,10 @@ static void planGroup(CommGroup* g) {
   int64_t chunkBytes, sliceBytes;
   if (g->proto == kProtoDirect) {
     // no FIFO: the chunk is only the interleaving grain of the sweeps (small grains keep all workgroups
-    // inside one compact address window per buffer)
-    chunkBytes = roundUp64(std::max<int64_t>(envInt("DFCCL_DIRECT_CHUNK_BYTES", 8 << 10), kAlignBytes), kAlignBytes);
+    // inside one compact address window per buffer).  8 KiB up to 256 MiB per rank, 32 KiB from there on
+    // (measured with 8 ranks: at 64 MiB 8 KiB tiles are 10 % faster than 32 KiB ones, at 256 MiB 15 % slower).
+    const int64_t tileDefault = (nBytes >= ((int64_t)256 << 20)) ? (32 << 10) : (8 << 10);
+    chunkBytes = roundUp64(std::max<int64_t>(envInt("DFCCL_DIRECT_CHUNK_BYTES", tileDefault), kAlignBytes), kAlignBytes);
     sliceBytes = chunkBytes;
     g->slicesPerChunk = 1;
     g->fifoSlots = 1;
@@ -515,6 +558,11 @@ static void planGroup(CommGroup* g) {
   if (g->device >= 0 && g->device < 64) sharers = std::max(sharers, gLiveRankCtxs[g->device].load());
   sharers = std::max(1, sharers);
   const int capacity = deviceWorkgroupSlots(g->device);
+  g->capacityUnknown = capacity <= 0;
+  if (g->capacityUnknown) {
+    fprintf(stderr, "dfccl: cannot tell how many daemon workgroups device %d keeps resident; not planning\n", g->device);
+    return;
+  }
   const int headroom = (int)std::min<int64_t>(std::max<int64_t>(0, envInt("DFCCL_RESIDENCY_HEADROOM", 8)), capacity / 2);
   int share = std::max(1, (capacity - headroom) / sharers);
   while (share > 1 && sharers * ((share + 7) & ~7) > capacity) share--;
@@ -580,16 +628,18 @@ static ncclResult_t prepareColl(int kind, size_t count, int dtype, int op, int r
   Scale scale;
   scale.kind = kScaleNone;
   scale.bits = 0;
+  uint64_t scalePtr = 0;
   if (reduces && op == ncclAvg) {
     devOp = ncclSum;
     scale = dfcclAvgScale(dtype, g->nRanks);
   } else if (reduces && op >= ncclNumOps) {
     auto it = comm->userOps.find(op - (int)ncclNumOps);
     if (it == comm->userOps.end()) return ncclInvalidArgument;
-    if (it->second.first != dtype) return ncclInvalidArgument;  // made for another datatype (enqueue.cc:1361-1365)
+    if (it->second.datatype != dtype) return ncclInvalidArgument;  // made for another datatype (enqueue.cc:1361-1365)
     devOp = ncclSum;
     scale.kind = kScalePre;
-    scale.bits = it->second.second;
+    scale.bits = it->second.bits;
+    scalePtr = it->second.devPtr;
   } else if (op >= ncclNumOps) {
     return ncclInvalidArgument;
   }
@@ -602,17 +652,21 @@ static ncclResult_t prepareColl(int kind, size_t count, int dtype, int op, int r
       g->dtypeUser = dtype;
       g->op = devOp;
       g->scaleKind = scale.kind;
-      g->scaleBits = scale.bits;
+      g->scaleBits.assign((size_t)g->nRanks, 0);
+      g->scalePtr.assign((size_t)g->nRanks, 0);
       g->root = root;
       g->countUser = count;
       planGroup(g);
+      if (g->capacityUnknown) return ncclUnhandledCudaError;  // (planned stays false: the next Prepare tries again)
       g->planned = true;
     } else if (g->kind != kind || g->dtypeUser != dtype || g->countUser != count || g->root != root ||
-               (reduces && (g->op != devOp || g->scaleKind != scale.kind || g->scaleBits != scale.bits))) {
-      // the ranks of a communicator must describe the same collective (for a PreMulSum operator that includes
-      // the scalar: the virtual ranks fold each other's inputs, so one scalar serves the whole communicator)
+               (reduces && (g->op != devOp || g->scaleKind != scale.kind))) {
+      // the ranks of a communicator must describe the same collective (every rank may bring its own scalar to a
+      // PreMulSum, as in the reference, where each rank scales the input it reads itself)
       return ncclInvalidArgument;
     }
+    g->scaleBits[(size_t)comm->rank] = scale.bits;
+    g->scalePtr[(size_t)comm->rank] = scalePtr;
   }
   comm->registered = true;
   ctx->collIndex[collId] = (int16_t)ctx->colls.size();
@@ -831,20 +885,27 @@ DFCCL_API ncclResult_t ncclCommUserRank(const ncclComm_t comm, int* rank) {
   return ncclSuccess;
 }
 
-// A reduction operator that multiplies every input by *scalar before summing (src/nccl.h.in:169-180,
-// src/enqueue.cc:1443-1490).  The scalar is read now (ncclScalarHostImmediate); one that lives in device memory
-// and is read while the collective runs is not supported on this path, where a collective is prepared once and
-// run many times.
+// A reduction operator that multiplies every input by *scalar before summing (src/nccl.h.in:148-180,
+// src/enqueue.cc:1443-1490).  ncclScalarHostImmediate: the scalar is read now.  ncclScalarDevice: `scalar` is a
+// device address, kept as it is (enqueue.cc:1470-1472) and dereferenced on the device whenever an instance of a
+// collective prepared with the operator starts (the reference dereferences it when the kernel starts on the
+// work element, src/collectives/device/common.h:117-136); the memory has to stay valid, and hold an element of
+// `datatype` at its natural alignment, for as long as the collective is registered.
 DFCCL_API ncclResult_t ncclRedOpCreatePreMulSum(ncclRedOp_t* op, void* scalar, ncclDataType_t datatype,
                                                 ncclScalarResidence_t residence, ncclComm_t comm) {
   if (op == nullptr || scalar == nullptr || comm == nullptr) return ncclInvalidArgument;
   const int es = typeSizeOf((int)datatype);
   if (es == 0) return ncclInvalidArgument;
-  if (residence != ncclScalarHostImmediate) return ncclInvalidArgument;
-  uint64_t bits = 0;
-  memcpy(&bits, scalar, (size_t)es);
+  if (residence != ncclScalarHostImmediate && residence != ncclScalarDevice) return ncclInvalidArgument;
+  uint64_t bits = 0, devPtr = 0;
+  if (residence == ncclScalarHostImmediate) {
+    memcpy(&bits, scalar, (size_t)es);
+  } else {
+    devPtr = (uint64_t)(uintptr_t)scalar;
+    if ((devPtr & ~kPtrMask) != 0 || devPtr % (uint64_t)es != 0) return ncclInvalidArgument;
+  }
   const int ix = comm->nextUserOp++;
-  comm->userOps[ix] = std::make_pair((int)datatype, bits);
+  comm->userOps[ix] = ncclComm::UserOp{(int)datatype, bits, devPtr};
   *op = (ncclRedOp_t)((int)ncclNumOps + ix);
   return ncclSuccess;
 }
@@ -949,7 +1010,18 @@ DFCCL_API ncclResult_t ofcclFinalizeRankCtx7StartHostThrds(ofcclRankCtx_t c) {
     p.slotBytes = g->slotBytes; p.fifoChanStride = g->chanStride;
     p.sendFifo = g->fifo ? g->fifo + (size_t)rank * g->nChannels * g->chanStride : nullptr;
     p.recvFifo = g->fifo ? g->fifo + (size_t)prev * g->nChannels * g->chanStride : nullptr;
-    p.proto = g->proto; p.scaleKind = g->scaleKind; p.scaleBits = g->scaleBits; p.pubs = g->pubs; p.p1 = g->p1;
+    p.proto = g->proto; p.scaleKind = g->scaleKind; p.pubs = g->pubs; p.p1 = g->p1;
+    p.scaleBits = g->scaleBits[(size_t)rank];
+    p.scalePtr = (const void*)(uintptr_t)g->scalePtr[(size_t)rank];
+    if (g->proto == kProtoDirect && g->scaleKind == kScalePre && p.scalePtr == nullptr) {
+      // the peers fold this rank's input: they find its scalar next to its buffer pointers.  Only the `scale`
+      // words of this rank's row are written (nothing has been announced through them yet).
+      std::vector<PeerPub> row((size_t)g->nChannels);
+      memset(row.data(), 0, row.size() * sizeof(PeerPub));
+      for (auto& e : row) e.scale = p.scaleBits;
+      HIPCHECK(hipMemcpy(g->pubs + (size_t)rank * g->nChannels, row.data(), row.size() * sizeof(PeerPub),
+                         hipMemcpyHostToDevice));
+    }
     p.loopsPerInstance = g->loopsPerInstance;
     p.lastChunkElems = g->lastChunkElems;
     p.tileCtr = g->tileCtrs ? g->tileCtrs + (size_t)rank * 16 : nullptr;
@@ -1143,8 +1215,18 @@ DFCCL_API ncclResult_t ofcclRunBcast(void* buff, int collId, CallbackFunc callba
 
 DFCCL_API ncclResult_t dfcclGetStats(ofcclRankCtx_t c, dfcclStats* out) {
   if (c == nullptr || out == nullptr) return ncclInvalidArgument;
+  // the caller says how large its structure is: nothing is written beyond that
+  const uint64_t callerBytes = out->structBytes;
+  if (callerBytes < 16 || callerBytes > 4096) return ncclInvalidArgument;
+  dfcclStats full;
+  dfcclStats* const user = out;
+  out = &full;
   memset(out, 0, sizeof(*out));
-  if (!c->finalized) return ncclInvalidUsage;
+  out->structBytes = std::min<uint64_t>(callerBytes, sizeof(dfcclStats));
+  if (!c->finalized) {
+    memcpy(user, out, (size_t)out->structBytes);
+    return ncclInvalidUsage;
+  }
   Daemon* d = c->daemon;
   {
     // A resident daemon writes its counters on request: raise the request number (the word after the control
@@ -1182,8 +1264,11 @@ DFCCL_API ncclResult_t dfcclGetStats(ofcclRankCtx_t c, dfcclStats* out) {
     out->slicesMoved += __atomic_load_n(&s->slicesMoved, __ATOMIC_ACQUIRE);
   }
   out->sqFullWaits = c->sqFullSpins.load(std::memory_order_relaxed);
-  std::lock_guard<std::mutex> lk(d->mu);
-  out->daemonLaunches = d->launches;
+  {
+    std::lock_guard<std::mutex> lk(d->mu);
+    out->daemonLaunches = d->launches;
+  }
+  memcpy(user, out, (size_t)out->structBytes);
   return ncclSuccess;
 }
 

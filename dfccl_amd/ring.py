@@ -23,13 +23,16 @@ class VirtualRing:
         self.finalized = False
 
     # -- registration -----------------------------------------------------------
-    def prepare(self, coll_id, kind, count, dtype, op=api.ncclSum, root=0, premul=None):
-        """premul: the bytes of one element; every rank then makes a PreMulSum operator with that scalar on its
-        communicator handle and registers the collective with it (op is ignored)."""
+    def prepare(self, coll_id, kind, count, dtype, op=api.ncclSum, root=0, premul=None, premul_device=None):
+        """premul: the bytes of one element, or a list with one such scalar per rank; every rank then makes a
+        PreMulSum operator with its scalar on its communicator handle and registers the collective with it (op is
+        ignored).  premul_device: a list with one device address per rank instead (ncclScalarDevice)."""
         comms = api.VirtualComm.create_all(self.n)
         for r, ctx in enumerate(self.ctxs):
-            if premul is not None:
-                op = comms[r].create_premul_sum(dtype, premul)
+            if premul_device is not None:
+                op = comms[r].create_premul_sum(dtype, device_ptr=premul_device[r])
+            elif premul is not None:
+                op = comms[r].create_premul_sum(dtype, premul[r] if isinstance(premul, (list, tuple)) else premul)
             if kind == "all_reduce":
                 ctx.prepare_all_reduce(count, dtype, op, comms[r], coll_id)
             elif kind == "reduce_scatter":

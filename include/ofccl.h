@@ -88,11 +88,15 @@ const char* ncclGetErrorString(ncclResult_t result);                            
  * *scalar (one element of `datatype`) before summing, for collectives prepared
  * on `comm` with that datatype (src/enqueue.cc:1443-1490; device semantics
  * src/include/reduce_kernel.h:503-668: one rounded multiply in the element type).
- * Differences on this path: the scalar is read when the operator is created
- * (ncclScalarHostImmediate; ncclScalarDevice returns ncclInvalidArgument,
- * because a collective is prepared once and run many times), and all ranks of
- * a communicator must give the same scalar (the virtual ranks fold each
- * other's inputs): Prepare returns ncclInvalidArgument otherwise.
+ * Every rank makes its own operator and may give its own scalar: rank r's
+ * input enters the sum multiplied by rank r's scalar.  With
+ * ncclScalarHostImmediate the scalar is read when the operator is created;
+ * with ncclScalarDevice `scalar` is a device address (aligned to the element
+ * size) that is dereferenced on the device whenever an instance of a
+ * collective prepared with the operator starts, so the memory has to stay
+ * valid while the collective is registered, and a new value takes effect with
+ * the next ofcclRun* (src/collectives/device/common.h:117-136 dereferences it
+ * when the kernel starts on the work element).
  * ncclAvg needs none of this: Prepare turns it into a sum that is divided by
  * the number of ranks afterwards (integer types, C++ integer division) or
  * whose inputs are multiplied by 1/nranks first (float types), as
@@ -189,6 +193,7 @@ ncclResult_t dfcclReduceCopy(const void* const* srcs, int nsrcs, void* dst, size
  * src/include/collectives_ofccl.h:173-179, enqueue_ofccl_dev.cu:1148) ------ */
 
 typedef struct {
+  uint64_t structBytes;     /* in: sizeof(dfcclStats) as the caller knows it; the library writes no more than that */
   uint64_t sqesRead;        /* submissions taken from the queue              */
   uint64_t cqesWritten;     /* completions posted                            */
   uint64_t ctxSaves;        /* preemptions: contexts saved to HBM            */
@@ -201,7 +206,10 @@ typedef struct {
 } dfcclStats;
 
 /* Sums the counters over this rank's workgroups. Valid after Finalize; exact
- * once the rank is idle. */
+ * once the rank is idle.  Set stats->structBytes = sizeof(dfcclStats) before
+ * the call: counters added to the end of the structure by a later version of
+ * the library are then not written past the caller's copy
+ * (ncclInvalidArgument if it is smaller than the first counter's end). */
 ncclResult_t dfcclGetStats(ofcclRankCtx_t rankCtx, dfcclStats* stats);
 
 /* Host steady-clock times (ns) of collId's last instance on this rank: when its

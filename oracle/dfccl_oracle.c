@@ -212,9 +212,14 @@ static void apply_range(int dtype, int op, const void* a, const void* b, void* o
 
 typedef struct {
   int base;      /* ORC_SUM..ORC_MIN: the op applied between elements */
-  int pre;       /* multiply every input by `scalar` (bits of one element) first */
+  int pre;       /* multiply every input by a scalar (bits of one element) first */
   int post;      /* divide the final value by (int)scalar */
   uint64_t scalar;
+  /* PreMulSum with one scalar per rank: every rank makes its own operator, and the multiplication is applied
+   * to a rank's input where that rank reads it (preOp on the user-input source of the rank's own primitives,
+   * src/collectives_ofccl/device/ofccl_prims_simple.h:405-411), so input r is scaled by rank r's scalar.
+   * NULL: `scalar` serves every rank. */
+  const uint64_t* per_rank;
 } orc_xop;
 
 uint64_t orc_avg_scalar(int dtype, int n) {
@@ -232,7 +237,7 @@ uint64_t orc_avg_scalar(int dtype, int n) {
 
 /* resolves a public op code (+ scalar for ORC_PREMULSUM, group size for ORC_AVG); returns 0 if valid */
 static int resolve_op(int dtype, int op, uint64_t scalar, int n, orc_xop* x) {
-  x->base = op; x->pre = 0; x->post = 0; x->scalar = 0;
+  x->base = op; x->pre = 0; x->post = 0; x->scalar = 0; x->per_rank = NULL;
   if (op >= ORC_SUM && op <= ORC_MIN) return 0;
   x->base = ORC_SUM;
   if (op == ORC_AVG) {
@@ -271,11 +276,19 @@ void orc_scale_apply(int dtype, int how, uint64_t scalar, void* buf, size_t n) {
   else if (how == 2) postdiv_range(dtype, scalar, buf, n);
 }
 
-/* a rank's input as it enters the reduction: the buffer itself, or a scaled copy in tmp */
-static const void* entering(int dtype, const orc_xop* x, const void* in, void* tmp, size_t n) {
+/* rank r's input as it enters the reduction: the buffer itself, or a copy in tmp scaled by r's scalar */
+static const void* entering(int dtype, const orc_xop* x, int r, const void* in, void* tmp, size_t n) {
   if (!x->pre) return in;
-  premul_range(dtype, x->scalar, in, tmp, n);
+  premul_range(dtype, x->per_rank ? x->per_rank[r] : x->scalar, in, tmp, n);
   return tmp;
+}
+
+/* the same resolution with one scalar per rank for ORC_PREMULSUM (scalars may be NULL for every other op) */
+static int resolve_op_r(int dtype, int op, const uint64_t* scalars, int n, orc_xop* x) {
+  if (op == ORC_PREMULSUM && scalars == NULL) return -1;
+  if (resolve_op(dtype, op, 0, n, x) != 0) return -1;
+  if (op == ORC_PREMULSUM) x->per_rank = scalars;
+  return 0;
 }
 
 /* ------------------------------------------------------------- reduce-copy */
@@ -292,11 +305,11 @@ static void reduce_copy_range(int dtype, const orc_xop* x, int k, const void* co
    * user input here, so a pre-multiplication applies to each of them. */
   void* tmp = x->pre ? malloc(n * s + 1) : NULL;
   void* tmp0 = x->pre ? malloc(n * s + 1) : NULL;
-  const void* first = entering(dtype, x, (const char*)srcs[0] + begin * s, tmp0, n);
+  const void* first = entering(dtype, x, 0, (const char*)srcs[0] + begin * s, tmp0, n);
   if (k == 1) memmove(d, first, n * s);
-  else apply_range(dtype, x->base, first, entering(dtype, x, (const char*)srcs[1] + begin * s, tmp, n), d, n);
+  else apply_range(dtype, x->base, first, entering(dtype, x, 1, (const char*)srcs[1] + begin * s, tmp, n), d, n);
   for (int j = 2; j < k; j++)
-    apply_range(dtype, x->base, d, entering(dtype, x, (const char*)srcs[j] + begin * s, tmp, n), d, n);
+    apply_range(dtype, x->base, d, entering(dtype, x, j, (const char*)srcs[j] + begin * s, tmp, n), d, n);
   if (x->post) postdiv_range(dtype, x->scalar, d, n);
   free(tmp);
   free(tmp0);
@@ -386,8 +399,16 @@ int orc_all_reduce(int dtype, int op, const orc_geom* g, int64_t count, const vo
 
 int orc_all_reduce_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t count, const void* const* send,
                      void* const* recv) {
+  uint64_t same[ORC_MAX_RANKS];
+  if (!geom_ok(g) || g->n_ranks > ORC_MAX_RANKS) return -1;
+  for (int r = 0; r < g->n_ranks; r++) same[r] = scalar;
+  return orc_all_reduce_xr(dtype, op, same, g, count, send, recv);
+}
+
+int orc_all_reduce_xr(int dtype, int op, const uint64_t* scalars, const orc_geom* g, int64_t count,
+                      const void* const* send, void* const* recv) {
   orc_xop x;
-  if (!geom_ok(g) || orc_type_size(dtype) == 0 || resolve_op(dtype, op, scalar, g->n_ranks, &x) != 0) return -1;
+  if (!geom_ok(g) || orc_type_size(dtype) == 0 || resolve_op_r(dtype, op, scalars, g->n_ranks, &x) != 0) return -1;
   const int n = g->n_ranks;
   const size_t s = (size_t)orc_type_size(dtype);
   if (n == 1) { /* one rank: a copy, with the scaling a sum of one term still gets */
@@ -422,7 +443,7 @@ int orc_all_reduce_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int6
           if (nelem < 0) nelem = 0;
           const char* in = (const char*)send[r] + (size_t)off * s;
           char* out = (char*)recv[r] + (size_t)off * s;
-          if (step <= n - 1) in = entering(dtype, &x, in, tmp, (size_t)nelem); /* the steps that read the user's input */
+          if (step <= n - 1) in = entering(dtype, &x, r, in, tmp, (size_t)nelem); /* the steps that read the user's input */
           if (step == 0) { /* send */
             memcpy(cur[r].data, in, (size_t)nelem * s);
           } else if (step <= n - 2) { /* recvReduceSend */
@@ -466,8 +487,16 @@ int orc_reduce_scatter(int dtype, int op, const orc_geom* g, int64_t recvcount, 
 
 int orc_reduce_scatter_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t recvcount,
                          const void* const* send, void* const* recv) {
+  uint64_t same[ORC_MAX_RANKS];
+  if (!geom_ok(g) || g->n_ranks > ORC_MAX_RANKS) return -1;
+  for (int r = 0; r < g->n_ranks; r++) same[r] = scalar;
+  return orc_reduce_scatter_xr(dtype, op, same, g, recvcount, send, recv);
+}
+
+int orc_reduce_scatter_xr(int dtype, int op, const uint64_t* scalars, const orc_geom* g, int64_t recvcount,
+                          const void* const* send, void* const* recv) {
   orc_xop x;
-  if (!geom_ok(g) || orc_type_size(dtype) == 0 || resolve_op(dtype, op, scalar, g->n_ranks, &x) != 0) return -1;
+  if (!geom_ok(g) || orc_type_size(dtype) == 0 || resolve_op_r(dtype, op, scalars, g->n_ranks, &x) != 0) return -1;
   const int n = g->n_ranks;
   const size_t s = (size_t)orc_type_size(dtype);
   if (n == 1) {
@@ -500,7 +529,7 @@ int orc_reduce_scatter_x(int dtype, int op, uint64_t scalar, const orc_geom* g, 
           else if (step <= n - 2) dest = (r + n - (step + 1)) % n;
           else dest = r;
           const int64_t off = chunk_off + (int64_t)dest * recvcount;
-          const char* in = entering(dtype, &x, (const char*)send[r] + (size_t)off * s, tmp, (size_t)nelem);
+          const char* in = entering(dtype, &x, r, (const char*)send[r] + (size_t)off * s, tmp, (size_t)nelem);
           if (step == 0) {
             memcpy(cur[r].data, in, (size_t)nelem * s);
           } else if (step <= n - 2) {
@@ -577,8 +606,16 @@ int orc_reduce(int dtype, int op, const orc_geom* g, int64_t count, int root, co
 
 int orc_reduce_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t count, int root,
                  const void* const* send, void* const* recv) {
+  uint64_t same[ORC_MAX_RANKS];
+  if (!geom_ok(g) || g->n_ranks > ORC_MAX_RANKS) return -1;
+  for (int r = 0; r < g->n_ranks; r++) same[r] = scalar;
+  return orc_reduce_xr(dtype, op, same, g, count, root, send, recv);
+}
+
+int orc_reduce_xr(int dtype, int op, const uint64_t* scalars, const orc_geom* g, int64_t count, int root,
+                  const void* const* send, void* const* recv) {
   orc_xop x;
-  if (!geom_ok(g) || orc_type_size(dtype) == 0 || resolve_op(dtype, op, scalar, g->n_ranks, &x) != 0) return -1;
+  if (!geom_ok(g) || orc_type_size(dtype) == 0 || resolve_op_r(dtype, op, scalars, g->n_ranks, &x) != 0) return -1;
   const int n = g->n_ranks;
   if (root < 0 || root >= n) return -1;
   const size_t s = (size_t)orc_type_size(dtype);
@@ -601,7 +638,7 @@ int orc_reduce_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t 
       /* the chain starts at the rank whose predecessor is the root and ends at the root */
       for (int k = 1; k <= n; k++) {
         const int r = (root + k) % n;
-        const char* in = entering(dtype, &x, (const char*)send[r] + (size_t)off * s, tmp, (size_t)nelem);
+        const char* in = entering(dtype, &x, r, (const char*)send[r] + (size_t)off * s, tmp, (size_t)nelem);
         if (k == 1) {
           memcpy(msg, in, (size_t)nelem * s); /* send */
         } else if (k < n) {

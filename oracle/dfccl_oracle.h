@@ -113,6 +113,17 @@ int orc_reduce_scatter_x(int dtype, int op, uint64_t scalar, const orc_geom* g, 
                          const void* const* send, void* const* recv);
 int orc_reduce_x(int dtype, int op, uint64_t scalar, const orc_geom* g, int64_t count, int root,
                  const void* const* send, void* const* recv);
+/* ... and with one scalar per rank (scalars[r] is rank r's): every rank makes its own PreMulSum operator
+ * (src/enqueue.cc:1443-1475) and the multiplication is applied to a rank's input by that rank's own primitives
+ * (preOp on the user-input source, src/collectives_ofccl/device/ofccl_prims_simple.h:405-411), so rank r's input
+ * enters the sum multiplied by rank r's scalar.  At most ORC_MAX_RANKS ranks. */
+#define ORC_MAX_RANKS 64
+int orc_all_reduce_xr(int dtype, int op, const uint64_t* scalars, const orc_geom* g, int64_t count,
+                      const void* const* send, void* const* recv);
+int orc_reduce_scatter_xr(int dtype, int op, const uint64_t* scalars, const orc_geom* g, int64_t recvcount,
+                          const void* const* send, void* const* recv);
+int orc_reduce_xr(int dtype, int op, const uint64_t* scalars, const orc_geom* g, int64_t count, int root,
+                  const void* const* send, void* const* recv);
 
 /* Ring position that owns element i of an all-reduce (does the last reduction
  * and so fixes the accumulation order). Closed form, independent of the

@@ -72,6 +72,10 @@ def lib():
         L.orc_all_reduce_x.argtypes = [ctypes.c_int, ctypes.c_int, u64, gp, ctypes.c_int64, vpp, vpp]
         L.orc_reduce_scatter_x.argtypes = [ctypes.c_int, ctypes.c_int, u64, gp, ctypes.c_int64, vpp, vpp]
         L.orc_reduce_x.argtypes = [ctypes.c_int, ctypes.c_int, u64, gp, ctypes.c_int64, ctypes.c_int, vpp, vpp]
+        u64p = ctypes.POINTER(u64)
+        L.orc_all_reduce_xr.argtypes = [ctypes.c_int, ctypes.c_int, u64p, gp, ctypes.c_int64, vpp, vpp]
+        L.orc_reduce_scatter_xr.argtypes = [ctypes.c_int, ctypes.c_int, u64p, gp, ctypes.c_int64, vpp, vpp]
+        L.orc_reduce_xr.argtypes = [ctypes.c_int, ctypes.c_int, u64p, gp, ctypes.c_int64, ctypes.c_int, vpp, vpp]
         L.orc_all_reduce_owner.argtypes = [gp, ctypes.c_int64, ctypes.c_int64]
         L.orc_cqe_encode.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.c_uint]
         L.orc_cqe_encode.restype = ctypes.c_uint64
@@ -123,10 +127,19 @@ def scalar_bits(dtype, value):
     return int(np.frombuffer(a.tobytes().ljust(8, b"\0"), dtype=np.uint64)[0])
 
 
+def _scalars(scalar, n):
+    """`scalar` of the reducing collectives: the bits of one element for every rank, or a sequence with one per
+    rank (every rank's own PreMulSum operator)."""
+    vals = list(scalar) if isinstance(scalar, (list, tuple)) else [scalar] * n
+    assert len(vals) == n
+    return (ctypes.c_uint64 * n)(*[int(v) for v in vals])
+
+
 def all_reduce(dtype, op, geom, sends, scalar=0):
     _check(dtype, sends)
     recvs = [np.zeros_like(s) for s in sends]
-    rc = lib().orc_all_reduce_x(dtype, op, scalar, ctypes.byref(geom), sends[0].size, _ptrs(sends), _ptrs(recvs))
+    rc = lib().orc_all_reduce_xr(dtype, op, _scalars(scalar, len(sends)), ctypes.byref(geom), sends[0].size,
+                                 _ptrs(sends), _ptrs(recvs))
     assert rc == 0
     return recvs
 
@@ -136,7 +149,8 @@ def reduce_scatter(dtype, op, geom, sends, scalar=0):
     n = geom.n_ranks
     recvcount = sends[0].size // n
     recvs = [np.zeros(recvcount, dtype=s.dtype) for s in sends]
-    rc = lib().orc_reduce_scatter_x(dtype, op, scalar, ctypes.byref(geom), recvcount, _ptrs(sends), _ptrs(recvs))
+    rc = lib().orc_reduce_scatter_xr(dtype, op, _scalars(scalar, len(sends)), ctypes.byref(geom), recvcount,
+                                     _ptrs(sends), _ptrs(recvs))
     assert rc == 0
     return recvs
 
@@ -153,7 +167,8 @@ def all_gather(dtype, geom, sends):
 def reduce(dtype, op, geom, root, sends, scalar=0):
     _check(dtype, sends)
     recvs = [np.zeros_like(s) for s in sends]
-    rc = lib().orc_reduce_x(dtype, op, scalar, ctypes.byref(geom), sends[0].size, root, _ptrs(sends), _ptrs(recvs))
+    rc = lib().orc_reduce_xr(dtype, op, _scalars(scalar, len(sends)), ctypes.byref(geom), sends[0].size, root,
+                             _ptrs(sends), _ptrs(recvs))
     assert rc == 0
     return recvs
 

@@ -13,6 +13,8 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
     if EMULATION_LIB:
         _enter_emulation()
+    elif _have_gpu():
+        _refuse_unvalidated_daemon_on_a_gpu(config)
 
 
 # DFCCL_TESTS_ON_EMULATION=<path of libdfccl_emul.so> (see tests/emul): the tests marked `gpu` that go through the
@@ -49,6 +51,28 @@ def _enter_emulation():
 
     torch.cuda.current_stream = lambda *a, **k: _NoStream()
     torch.cuda.synchronize = lambda *a, **k: None
+
+
+def _refuse_unvalidated_daemon_on_a_gpu(config):
+    """On a real GPU: the sources of the daemon kernel must be the ones the host emulation last validated
+    (tests/test_daemon_emulation.py records their hash when all its scenarios pass).  A record that names other
+    sources ends the session before anything is launched; DFCCL_UNVALIDATED_DAEMON_OK=1 overrides, and a missing
+    record (the CPU suite has not been run in this tree) only warns."""
+    if EMULATION_LIB or os.environ.get("DFCCL_UNVALIDATED_DAEMON_OK") == "1":
+        return
+    markexpr = getattr(config.option, "markexpr", "") or ""
+    if "gpu" not in markexpr or "not gpu" in markexpr:
+        return
+    stamp = os.path.join(ROOT, "tests", "emul", "validated_sources.stamp")
+    if not os.path.exists(stamp):
+        print("conftest: no record of an emulation run in this tree (tests/emul/validated_sources.stamp)", file=sys.stderr)
+        return
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from test_daemon_emulation import sources_hash
+    if open(stamp).read().strip() != sources_hash():
+        pytest.exit("the daemon's sources have changed since the host emulation last passed on them: run "
+                    "`python -m pytest tests/test_daemon_emulation.py` first (or set DFCCL_UNVALIDATED_DAEMON_OK=1)",
+                    returncode=3)
 
 
 def _have_gpu():

@@ -62,6 +62,15 @@ void barrierMismatch(int tid, int line, int line0) {
   abort();
 }
 
+void notUniform(int line, uint64_t mine, uint64_t first) {
+  fprintf(stderr,
+          "emul: NOT UNIFORM: block %u thread %u holds %#llx at the DFCCL_UNIFORM of line %d, lane 0 of its wave holds "
+          "%#llx\n",
+          tls.bIdx.x, tls.tIdx.x, (unsigned long long)mine, line, (unsigned long long)first);
+  fflush(stderr);
+  abort();
+}
+
 void* wgSharedMem(size_t bytes) {
   Workgroup* wg = tls.wg;
   if (bytes > sizeof(wg->lds)) {

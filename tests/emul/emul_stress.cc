@@ -187,6 +187,7 @@ static int scenarioRepeat(int n, int count, int reps, int ncolls) {
     }
   }
   dfcclStats st;
+  st.structBytes = sizeof(st);
   uint64_t saves = 0, cqes = 0;
   for (int r = 0; r < n; r++) {
     CHECK(dfcclGetStats(ring.ctxs[r], &st));
@@ -309,6 +310,7 @@ static int scenarioRelaunch(int n) {
     if (round == 0) sleep(3);  // idle: every workgroup leaves
   }
   dfcclStats st;
+  st.structBytes = sizeof(st);
   CHECK(dfcclGetStats(ring.ctxs[0], &st));
   ring.destroy();
   freeBuffers();
@@ -408,7 +410,12 @@ static int scenarioFuzz(uint64_t seed, int rounds) {
     return (x >> 11) % m;
   };
   const int n = 2 + (int)rnd(5), ncolls = 1 + (int)rnd(7);
-  struct Coll { int kind, count, root, dt, op; };
+  // op: ncclSum / ncclMax / ncclMin / ncclAvg, or kPreMul: every rank makes its own PreMulSum operator with the
+  // scalar (rank % 3) + 1, read from host memory when the operator is made or (premulDevice) from memory the
+  // daemon dereferences whenever an instance starts
+  constexpr int kPreMul = 100;
+  struct Coll { int kind, count, root, dt, op, premulDevice; };
+  auto scalarOf = [](int r) { return (r % 3) + 1; };
   std::vector<Coll> colls;
   Ring ring(n);
   for (int c = 0; c < ncolls; c++) {
@@ -419,13 +426,21 @@ static int scenarioFuzz(uint64_t seed, int rounds) {
     k.root = (int)rnd((uint64_t)n);
     k.dt = (int)rnd(10);
     const bool isFloat = k.dt == ncclFloat16 || k.dt == ncclFloat32 || k.dt == ncclFloat64 || k.dt == ncclBfloat16;
-    const int pick = (int)rnd(3);
-    k.op = pick == 0 ? (int)ncclSum : pick == 1 ? (int)ncclMax : (isFloat ? (int)ncclMin : (int)ncclAvg);
+    const int pick = (int)rnd(4);
+    k.op = pick == 0 ? (int)ncclSum : pick == 1 ? (int)ncclMax : pick == 2 ? (isFloat ? (int)ncclMin : (int)ncclAvg) : kPreMul;
+    k.premulDevice = (int)rnd(2);
     colls.push_back(k);
     auto& comms = ring.newComms();
     const ncclDataType_t dt = (ncclDataType_t)k.dt;
-    const ncclRedOp_t op = (ncclRedOp_t)k.op;
     for (int r = 0; r < n; r++) {
+      ncclRedOp_t op = (ncclRedOp_t)k.op;
+      if (k.op == kPreMul) {
+        // one element of the type holding the rank's scalar (the buffer lives as long as the run: the daemon reads
+        // it at every instance when the operator was made with ncclScalarDevice)
+        char* scalar = exactAlloc((size_t)elemSize(k.dt));
+        putElem(scalar, 0, k.dt, scalarOf(r));
+        CHECK(ncclRedOpCreatePreMulSum(&op, scalar, dt, k.premulDevice ? ncclScalarDevice : ncclScalarHostImmediate, comms[r]));
+      }
       switch (k.kind) {
         case 0: CHECK(ofcclPrepareAllReduce(k.count, dt, op, comms[r], c, ring.ctxs[r])); break;
         case 1: CHECK(ofcclPrepareReduceScatter(k.count, dt, op, comms[r], c, ring.ctxs[r])); break;
@@ -447,14 +462,16 @@ static int scenarioFuzz(uint64_t seed, int rounds) {
     }
   auto val = [](int c, int r, int i, int rep) { return (i * 31 + r * 5 + c * 7 + rep * 3) % 4; };
   auto reduce = [&](int c, int i, int rep) {  // the reduction of element i over the ranks
-    int acc = 0, mx = 0, mn = 1 << 30;
+    int acc = 0, mx = 0, mn = 1 << 30, scaled = 0;
     for (int q = 0; q < n; q++) {
       const int v = val(c, q, i, rep);
       acc += v;
+      scaled += v * scalarOf(q);  // (at most 6 ranks x 3 x 3: exact in every element type)
       mx = v > mx ? v : mx;
       mn = v < mn ? v : mn;
     }
     switch (colls[c].op) {
+      case kPreMul: return scaled;
       case ncclSum: return acc;
       case ncclMax: return mx;
       case ncclMin: return mn;
@@ -595,6 +612,7 @@ static int scenarioBackpressure(int n, int ncolls, int rounds, int cbSleepUs) {
       }
   uint64_t fullWaits = 0, cqes = 0;
   dfcclStats st;
+  st.structBytes = sizeof(st);
   for (int r = 0; r < n; r++) {
     CHECK(dfcclGetStats(ring.ctxs[r], &st));
     fullWaits += st.sqFullWaits;
@@ -671,6 +689,7 @@ static int scenarioTwoRings(int n) {
       }
     }
   dfcclStats st;
+  st.structBytes = sizeof(st);
   CHECK(dfcclGetStats(b.ctxs[0], &st));
   a.destroy();
   b.destroy();

@@ -137,6 +137,20 @@ inline T shflFrom(T v, int src, int line) {
   return out;
 }
 
+// A value the kernel declares to be the same in every lane of the wave (on the GPU it is moved to scalar
+// registers with v_readfirstlane, and the wave then branches on it as one): here every lane compares its own
+// value with lane 0's, and a lane that disagrees ends the run with both values and the source line.
+void notUniform(int line, uint64_t mine, uint64_t first);
+template <typename T>
+inline T uniformChecked(T v, int line) {
+  const T first = shflFrom(v, 0, line);
+  uint64_t a = 0, b = 0;
+  memcpy(&a, &v, sizeof(T));
+  memcpy(&b, &first, sizeof(T));
+  if (a != b) notUniform(line, a, b);
+  return first;
+}
+
 void* wgSharedMem(size_t bytes);  // the workgroup's LDS block (the same address for all its threads)
 
 struct Job;     // one kernel launch: its threads
@@ -151,6 +165,8 @@ void launch(Stream* s, unsigned grid, unsigned block, std::function<void()> body
 #define DFCCL_WAVE_LDS_SYNC() ::emul::waveSync(__LINE__)
 
 #define DFCCL_WAVE_UNIFORM(x) ::emul::shflFrom((x), 0, __LINE__)
+#define DFCCL_UNIFORM(x) ::emul::uniformChecked((x), __LINE__)
+#define DFCCL_FRESH_PER_ROUND(v) ((void)0)  // (a hint for the GPU compiler's register allocation)
 
 // EMUL_NEVER_LEAVE=1: the daemon's workgroups ignore every reason to leave (see DFCCL_TEST_NEVER_LEAVES in daemon.hip)
 namespace emul { extern bool gNeverLeave; }

@@ -58,6 +58,31 @@ CASES = [
     ("reduce_copy", orc.F16, orc.AVG, 3, 1000, 0, None),
 ]
 
+# PreMulSum with every rank's own scalar (rank r's input enters the sum times VALUES[r]):
+# kind, dtype, values per rank, n, count, root, geometry.  Arrays p<idx>_in<r> / p<idx>_out<r>.
+PREMUL_CASES = [
+    ("all_reduce", orc.F32, [0.3, -1.7, 2.5, 0.01], 4, 2048, 0, (1, 2048, 256)),
+    ("all_reduce", orc.BF16, [-1.5, 0.5, 2.0, -0.25, 1.0, 3.0, -2.0, 0.75], 8, 4100, 0, (1, 4096, 512)),
+    ("all_reduce", orc.I32, [1000003, -3, 7], 3, 1500, 0, (1, 2048, 256)),
+    ("all_reduce", orc.F64, [1e-3, -2.5], 2, 600, 0, (1, 1024, 128)),
+    ("reduce_scatter", orc.F16, [0.5, -1.25, 2.0, 0.1], 4, 700, 0, (1, 512, 512)),
+    ("reduce", orc.U8, [3, 2, 5], 3, 2000, 1, (1, 8192, 1024)),
+]
+
+
+def premul_bits(dtype, values):
+    return [orc.scalar_bits(dtype, v) for v in values]
+
+
+def run_premul_case(kind, dtype, values, n, count, root, geom, sends):
+    g = orc.Geom(n, *geom)
+    bits = premul_bits(dtype, values)
+    if kind == "all_reduce":
+        return orc.all_reduce(dtype, orc.PREMULSUM, g, sends, scalar=bits)
+    if kind == "reduce_scatter":
+        return orc.reduce_scatter(dtype, orc.PREMULSUM, g, sends, scalar=bits)
+    return orc.reduce(dtype, orc.PREMULSUM, g, root, sends, scalar=bits)
+
 
 def run_case(kind, dtype, op, n, count, root, geom, sends):
     if kind == "reduce_copy":
@@ -88,6 +113,14 @@ def main():
             out[f"c{idx}_in{r}"] = a
         for r, a in enumerate(recvs):
             out[f"c{idx}_out{r}"] = a
+    for idx, (kind, dtype, values, n, count, root, geom) in enumerate(PREMUL_CASES):
+        length = count * n if kind == "reduce_scatter" else count
+        sends = [datagen.make(dtype, 12000 + 16 * idx + r, length) for r in range(n)]
+        recvs = run_premul_case(kind, dtype, values, n, count, root, geom, sends)
+        for r, a in enumerate(sends):
+            out[f"p{idx}_in{r}"] = a
+        for r, a in enumerate(recvs):
+            out[f"p{idx}_out{r}"] = a
     np.savez_compressed(os.path.join(HERE, "ring_cases.npz"), **out)
     print("wrote", len(out), "arrays")
 

@@ -25,6 +25,26 @@ SAN = os.environ.get("EMUL_SAN", "none")
 SLOW = 1 if SAN == "none" else 8
 
 
+# Which sources the emulation has validated: when every test of this file has passed in one session, the hash of
+# the kernel and runtime sources is recorded in tests/emul/validated_sources.stamp.  The GPU suite refuses to start
+# on a real GPU while that record names other sources (tests/conftest.py): a persistent kernel that goes wrong hangs
+# or faults the GPU, so no build of it goes there before it has run here.
+STAMP = os.path.join(EMUL, "validated_sources.stamp")
+PASSED = set()
+
+
+def sources_hash():
+    import hashlib
+    csrc = os.path.join(os.path.dirname(HERE), "dfccl_amd", "csrc")
+    files = sorted(os.path.join(csrc, f) for f in os.listdir(csrc) if f.endswith((".hip", ".h")))
+    files.append(os.path.join(os.path.dirname(HERE), "include", "ofccl.h"))
+    h = hashlib.sha256()
+    for f in files:
+        h.update(os.path.basename(f).encode() + b"\0")
+        h.update(open(f, "rb").read())
+    return h.hexdigest()
+
+
 @pytest.fixture(scope="module")
 def stress():
     r = subprocess.run(["make", "-C", EMUL, f"SAN={SAN}", "-j4"], capture_output=True, text=True, timeout=1800)
@@ -55,6 +75,9 @@ SCENARIOS = [
     ("repeat-tiny-budget-ragged", TINY, ["repeat", "3", "5000", "6", "2"]),
     ("repeat-8-ranks", {}, ["repeat", "8", "2048", "4", "1"]),
     ("repeat-several-channels", {"NCCL_MAX_NCHANNELS": "8"}, ["repeat", "2", "300000", "2", "1"]),
+    # the traced build of the kernel (DFCCL_TRACE=1): same scheduler, with the timeline stamps compiled in
+    ("repeat-traced", {"DFCCL_TRACE": "1", "DFCCL_TRACE_FILE": "/dev/null"}, ["repeat", "4", "2048", "6", "2"]),
+    ("mixed-fifo-traced", {"DFCCL_TRACE": "1", "DFCCL_TRACE_FILE": "/dev/null", "DFCCL_PROTO": "fifo"}, ["mixed", "3", "1"]),
     # all five collectives side by side, ranks submit in different orders
     ("mixed-direct", {}, ["mixed", "4", "2"]),
     ("mixed-direct-tiny-budget", TINY, ["mixed", "4", "2"]),
@@ -99,6 +122,7 @@ def test_emulated_daemon(stress, name, env, args):
     assert r.returncode == 0, f"{name}: rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
     assert " ok" in r.stdout
     assert no_sanitizer_report(r), r.stderr[-6000:]
+    PASSED.add(name)
 
 
 def test_a_daemon_that_never_leaves_ends_the_process_with_a_report(stress):
@@ -113,6 +137,7 @@ def test_a_daemon_that_never_leaves_ends_the_process_with_a_report(stress):
     assert r.returncode == 70, f"rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
     assert "still resident after an abort request" in r.stderr
     assert "ofcclDestroy returned" not in r.stdout
+    PASSED.add("stuck")
 
 
 DRIVER_ENV = {"disorder-small-queue": {"DFCCL_SQ_CAPACITY": "4"}}
@@ -149,6 +174,7 @@ def test_emulated_daemon_under_the_native_driver(stress, name, args):
         assert out["deadlocks"] == 0
     if name == "disorder-small-queue":
         assert out["sq_full_waits"] > 0 and out["cqes"] == 3 * 24
+    PASSED.add("driver-" + name)
 
 
 @pytest.mark.skipif(SAN != "none", reason="python cannot load a sanitizer build of the library without its runtime preloaded")
@@ -164,7 +190,7 @@ def test_parity_tests_on_the_emulation(stress):
               "EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "120"})
     pick = ("test_small_all_reduce_and_in_place or test_in_place_and_absent_buffers or golden or "
             "test_other_collectives_disordered or test_rank_by_rank or forced_preemption or avg_small_and_ragged or "
-            "premul_sum_operator or nan_operands")
+            "premul_sum or nan_operands")
     r = subprocess.run([sys.executable, "-m", "pytest", os.path.join(HERE, "test_daemon_gpu.py"),
                         os.path.join(HERE, "test_golden.py"), "-q", "-m", "gpu", "-x", "-p", "no:cacheprovider",
                         "--timeout", "600", "-k", pick], env=e, capture_output=True, text=True, timeout=1200,
@@ -172,3 +198,17 @@ def test_parity_tests_on_the_emulation(stress):
     tail = r.stdout[-3000:] + r.stderr[-2000:]
     assert r.returncode == 0, tail
     assert " passed" in r.stdout and " failed" not in r.stdout, tail
+    PASSED.add("parity")
+
+
+def test_zz_record_the_sources_the_emulation_has_validated():
+    """Last in this file: if every scenario above has passed in this session (none deselected), the sources they
+    ran are recorded as validated."""
+    want = {s[0] for s in SCENARIOS} | {"stuck"} | {"driver-" + d[0] for d in DRIVER}
+    if SAN == "none":
+        want.add("parity")
+    missing = want - PASSED
+    if missing:
+        pytest.skip(f"not every scenario ran in this session (missing: {sorted(missing)[:4]}...): no record written")
+    with open(STAMP, "w") as f:
+        f.write(sources_hash() + "\n")

@@ -136,17 +136,30 @@ def test_avg_small_and_ragged(n, count):
     check("all_reduce", orc.I8, orc.AVG, n, count, seed=261)
 
 
-@pytest.mark.parametrize("dtype,value", [(orc.F32, 0.3), (orc.BF16, -1.5), (orc.F64, 1e-3), (orc.I32, 1000003),
-                                         (orc.U8, 3)])
-def test_premul_sum_operator(dtype, value):
-    # an operator made by ncclRedOpCreatePreMulSum: every input times the scalar (one rounding in the type), summed
+PREMUL_VALUES = {orc.F32: [0.3, -1.7, 2.5, 0.01, 1.0, -0.5, 3.25, 0.125], orc.BF16: [-1.5, 0.5, 2.0, -0.25, 1.0, 3.0, -2.0, 0.75],
+                 orc.F64: [1e-3, -2.5, 0.3, 7.0, 1.0, -1.0, 0.5, 2.0], orc.F16: [0.5, -1.25, 2.0, 0.1, 1.0, -3.0, 0.25, 1.5],
+                 orc.I32: [1000003, -3, 7, 2, 1, -1, 5, 11], orc.U8: [3, 2, 5, 1, 7, 4, 6, 9],
+                 orc.I64: [-1000000007, 3, 2, 5, 1, -1, 7, 11]}
+
+
+def scalar_bytes_of(dtype, value):
+    return int(orc.scalar_bits(dtype, value)).to_bytes(8, "little")[:orc.TYPE_SIZE[dtype]]
+
+
+@pytest.mark.parametrize("per_rank", [False, True], ids=["one-scalar", "scalar-per-rank"])
+@pytest.mark.parametrize("dtype", [orc.F32, orc.BF16, orc.F64, orc.I32, orc.U8])
+def test_premul_sum_operator(dtype, per_rank):
+    # operators made by ncclRedOpCreatePreMulSum, one per rank: every rank's input times that rank's scalar (one
+    # rounding in the type), summed in the ring's order; all three reducing collectives
     from dfccl_amd.ring import VirtualRing
-    n, count = 4, 70001
-    bits = orc.scalar_bits(dtype, value)
-    scalar_bytes = int(bits).to_bytes(8, "little")[:orc.TYPE_SIZE[dtype]]
+    n, count, root = 4, (9001 if gpu_util.EMULATED else 70001), 2
+    values = PREMUL_VALUES[dtype][:n] if per_rank else [PREMUL_VALUES[dtype][0]] * n
+    bits = [orc.scalar_bits(dtype, v) for v in values]
+    premul = [scalar_bytes_of(dtype, v) for v in values]
     with VirtualRing(n) as ring:
-        ring.prepare(0, "all_reduce", count, dtype, premul=scalar_bytes)
-        ring.prepare(1, "reduce_scatter", count // n, dtype, premul=scalar_bytes)
+        ring.prepare(0, "all_reduce", count, dtype, premul=premul)
+        ring.prepare(1, "reduce_scatter", count // n, dtype, premul=premul)
+        ring.prepare(2, "reduce", count, dtype, root=root, premul=premul)
         ring.finalize()
         sends_np, sends, recvs = make_buffers("all_reduce", dtype, n, count, 270)
         want = orc.all_reduce(dtype, orc.PREMULSUM, geom_of(ring, 0), sends_np, scalar=bits)
@@ -158,6 +171,85 @@ def test_premul_sum_operator(dtype, value):
         ring.run(1, rs_send, rs_recv, timeout=30)
         for r in range(n):
             assert np.array_equal(to_np(dtype, rs_recv[r]), want[r]), r
+        rd_np, rd_send, rd_recv = make_buffers("reduce", dtype, n, count, 290)
+        want = orc.reduce(dtype, orc.PREMULSUM, geom_of(ring, 2), root, rd_np, scalar=bits)
+        ring.run(2, rd_send, rd_recv, timeout=30)
+        assert np.array_equal(to_np(dtype, rd_recv[root]), want[root])
+
+
+@pytest.mark.parametrize("n,count", [(2, 1000), (8, 4099), (3, 200003)])
+def test_premul_sum_scalar_per_rank_small_and_large(n, count):
+    # sizes that wave 0 folds alone (2 and 8 ranks) and one that takes several channels
+    from dfccl_amd.ring import VirtualRing
+    if gpu_util.EMULATED:
+        count = min(count, 40003)
+    for dtype in (orc.F16, orc.I64):
+        values = PREMUL_VALUES[dtype][:n]
+        bits = [orc.scalar_bits(dtype, v) for v in values]
+        with VirtualRing(n) as ring:
+            ring.prepare(0, "all_reduce", count, dtype, premul=[scalar_bytes_of(dtype, v) for v in values])
+            ring.finalize()
+            sends_np, sends, recvs = make_buffers("all_reduce", dtype, n, count, 275)
+            want = orc.all_reduce(dtype, orc.PREMULSUM, geom_of(ring, 0), sends_np, scalar=bits)
+            for rep in range(2):
+                ring.run(0, sends, recvs, timeout=30)
+                for r in range(n):
+                    assert np.array_equal(to_np(dtype, recvs[r]), want[r]), (dtype, rep, r)
+
+
+@pytest.mark.parametrize("dtype", [orc.F32, orc.BF16, orc.I32, orc.F64, orc.U8])
+def test_premul_sum_scalar_in_device_memory(dtype):
+    # ncclScalarDevice: every rank's scalar lives in device memory and is read whenever an instance starts, so a
+    # value written between two runs takes effect with the second (src/collectives/device/common.h:117-136)
+    from dfccl_amd.ring import VirtualRing
+    n, count = 4, 30011
+    es = orc.TYPE_SIZE[dtype]
+    first, second = PREMUL_VALUES[dtype][:n], PREMUL_VALUES[dtype][n:2 * n]
+    # one element of the type per rank, 16 bytes apart
+    slots = torch.zeros(n * 16, dtype=torch.uint8, device=gpu_util.DEVICE)
+
+    def write(values):
+        host = np.zeros(n * 16, np.uint8)
+        for r, v in enumerate(values):
+            host[r * 16:r * 16 + es] = np.frombuffer(scalar_bytes_of(dtype, v), np.uint8)
+        slots.copy_(torch.from_numpy(host))
+        torch.cuda.current_stream().synchronize()
+
+    write(first)
+    with VirtualRing(n) as ring:
+        ring.prepare(0, "all_reduce", count, dtype, premul_device=[slots.data_ptr() + 16 * r for r in range(n)])
+        ring.prepare(1, "reduce_scatter", count // n, dtype,
+                     premul_device=[slots.data_ptr() + 16 * r for r in range(n)])
+        ring.finalize()
+        sends_np, sends, recvs = make_buffers("all_reduce", dtype, n, count, 295)
+        rs_np, rs_send, rs_recv = make_buffers("reduce_scatter", dtype, n, count // n, 296)
+        for values in (first, second):
+            write(values)
+            bits = [orc.scalar_bits(dtype, v) for v in values]
+            want = orc.all_reduce(dtype, orc.PREMULSUM, geom_of(ring, 0), sends_np, scalar=bits)
+            ring.run(0, sends, recvs, timeout=30)
+            for r in range(n):
+                assert np.array_equal(to_np(dtype, recvs[r]), want[r]), r
+            want = orc.reduce_scatter(dtype, orc.PREMULSUM, geom_of(ring, 1), rs_np, scalar=bits)
+            ring.run(1, rs_send, rs_recv, timeout=30)
+            for r in range(n):
+                assert np.array_equal(to_np(dtype, rs_recv[r]), want[r]), r
+
+
+def test_premul_sum_on_a_communicator_of_one_rank():
+    # a sum of one term is still multiplied, out of place and in place
+    from dfccl_amd.ring import VirtualRing
+    dtype, count = orc.F32, 5003
+    bits = orc.scalar_bits(dtype, 0.3)
+    with VirtualRing(1) as ring:
+        ring.prepare(0, "all_reduce", count, dtype, premul=scalar_bytes_of(dtype, 0.3))
+        ring.finalize()
+        sends_np, sends, recvs = make_buffers("all_reduce", dtype, 1, count, 297)
+        want = orc.all_reduce(dtype, orc.PREMULSUM, geom_of(ring, 0), sends_np, scalar=bits)
+        ring.run(0, sends, recvs, timeout=30)
+        assert np.array_equal(to_np(dtype, recvs[0]), want[0])
+        ring.run(0, sends, sends, timeout=30)
+        assert np.array_equal(to_np(dtype, sends[0]), want[0])
 
 
 def test_premul_sum_operator_errors():
@@ -177,11 +269,16 @@ def test_premul_sum_operator_errors():
         with pytest.raises(api.NcclError):
             ctxs[0].prepare_all_reduce(100, dfccl_amd.ncclFloat32, op0 + 17, comms[0], 0)
         ctxs[0].prepare_all_reduce(100, dfccl_amd.ncclFloat32, op0, comms[0], 0)
-        # the ranks of a communicator have to agree on the scalar
-        op1 = comms[1].create_premul_sum(dfccl_amd.ncclFloat32, np.array([0.25], np.float32).tobytes())
+        # the ranks of a communicator have to agree on the kind of operator (a scalar of their own is fine) ...
         with pytest.raises(api.NcclError) as e:
-            ctxs[1].prepare_all_reduce(100, dfccl_amd.ncclFloat32, op1, comms[1], 0)
+            ctxs[1].prepare_all_reduce(100, dfccl_amd.ncclFloat32, dfccl_amd.ncclSum, comms[1], 0)
         assert e.value.code == 4
+        # ... and a scalar in device memory has to be aligned to its type
+        with pytest.raises(api.NcclError) as e:
+            comms[1].create_premul_sum(dfccl_amd.ncclFloat32, device_ptr=0x7f0000000002)
+        assert e.value.code == 4
+        op1 = comms[1].create_premul_sum(dfccl_amd.ncclFloat32, np.array([0.25], np.float32).tobytes())
+        ctxs[1].prepare_all_reduce(100, dfccl_amd.ncclFloat32, op1, comms[1], 0)
         comms[0].destroy_op(op0)
         with pytest.raises(api.NcclError):
             comms[0].destroy_op(op0)

@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(HERE, "golden"))
 
 import dfccl_oracle as orc  # noqa: E402
-from make_golden import CASES, run_case  # noqa: E402
+from make_golden import CASES, PREMUL_CASES, run_case, run_premul_case  # noqa: E402
 
 DATA = np.load(os.path.join(HERE, "golden", "ring_cases.npz"), allow_pickle=False)
 
@@ -66,6 +66,50 @@ def test_hip_path_matches_golden(idx, monkeypatch):
         ring.run(0, sends, recvs, timeout=30)
         copy_kind = kind in ("all_gather", "broadcast")
         if not (copy_kind or order_independent(dtype, op) or same_geometry or kind in ("reduce_scatter", "reduce")):
+            pytest.skip("float all-reduce planned with another chunk geometry than the fixture's")
+        for r in range(n):
+            if kind == "reduce" and r != root:
+                continue
+            assert np.array_equal(to_np(dtype, recvs[r]), outs[r]), (idx, r)
+
+
+# ---- PreMulSum with a scalar per rank ------------------------------------------------------------------------
+
+def premul_arrays(idx, n):
+    return [DATA[f"p{idx}_in{r}"] for r in range(n)], [DATA[f"p{idx}_out{r}"] for r in range(n)]
+
+
+@pytest.mark.parametrize("idx", range(len(PREMUL_CASES)))
+def test_oracle_reproduces_golden_premul_sum(idx):
+    kind, dtype, values, n, count, root, geom = PREMUL_CASES[idx]
+    sends, outs = premul_arrays(idx, n)
+    got = run_premul_case(kind, dtype, values, n, count, root, geom, [s.copy() for s in sends])
+    for r in range(n):
+        assert np.array_equal(got[r], outs[r]), (idx, r)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("idx", range(len(PREMUL_CASES)))
+def test_hip_path_matches_golden_premul_sum(idx, monkeypatch):
+    import torch
+    from dfccl_amd.ring import VirtualRing
+    import gpu_util
+    from gpu_util import TORCH_OF, to_gpu, to_np
+    kind, dtype, values, n, count, root, geom = PREMUL_CASES[idx]
+    sends_np, outs = premul_arrays(idx, n)
+    sends = [to_gpu(dtype, s) for s in sends_np]
+    monkeypatch.setenv("DFCCL_DAEMON_MAX_MS", "10000")
+    recvs = [torch.zeros(count, dtype=TORCH_OF[dtype], device=gpu_util.DEVICE) for _ in range(n)]
+    torch.cuda.current_stream().synchronize()
+    es = orc.TYPE_SIZE[dtype]
+    premul = [int(orc.scalar_bits(dtype, v)).to_bytes(8, "little")[:es] for v in values]
+    with VirtualRing(n) as ring:
+        ring.prepare(0, kind, count, dtype, root=root, premul=premul)
+        ring.finalize()
+        g = ring.ctxs[0].geometry(0)
+        same_geometry = (g.nChannels, g.chunkElems, g.alignElems) == geom
+        ring.run(0, sends, recvs, timeout=30)
+        if kind == "all_reduce" and dtype in orc.FLOAT_DTYPES and not same_geometry:
             pytest.skip("float all-reduce planned with another chunk geometry than the fixture's")
         for r in range(n):
             if kind == "reduce" and r != root:

@@ -169,6 +169,72 @@ def test_reduce_scatter_and_reduce_premulsum_floats():
     assert np.array_equal(orc.reduce(orc.F32, orc.PREMULSUM, g, root, sends, scalar=s)[root], acc)
 
 
+# ---- PreMulSum with every rank's own scalar: input r enters the sum multiplied by rank r's scalar ------------
+# (every rank makes its own operator, src/enqueue.cc:1443-1475, and applies it to the input it reads itself,
+# src/collectives_ofccl/device/ofccl_prims_simple.h:405-411)
+
+PER_RANK_VALUES = [0.5, -1.25, 3.0, 0.0625, 1.5, -0.75, 2.0, 0.3]
+
+
+@pytest.mark.parametrize("dtype", orc.FLOAT_DTYPES)
+@pytest.mark.parametrize("n,C,chunk,align,count", GEOMS[:6])
+def test_premulsum_all_reduce_with_a_scalar_per_rank(dtype, n, C, chunk, align, count):
+    g = orc.Geom(n, C, chunk, align)
+    sends = [datagen.make(dtype, 1100 + r, count) for r in range(n)]
+    scalars = [orc.scalar_bits(dtype, PER_RANK_VALUES[r % 8] * (1 + r // 8)) for r in range(n)]
+    assert len(set(scalars)) == n  # all different: a scalar applied to the wrong rank's input would be noticed
+    scaled = [np_mul(dtype, sends[r], scalars[r]) for r in range(n)]
+    owner = py_owner(n, C, chunk, align, count)
+    want = np.empty_like(sends[0])
+    for c in range(n):
+        sel = owner == c
+        acc = scaled[(c + 1) % n][sel]
+        for j in range(2, n + 1):
+            acc = np_add(dtype, scaled[(c + j) % n][sel], acc)
+        want[sel] = acc
+    for got in orc.all_reduce(dtype, orc.PREMULSUM, g, sends, scalar=scalars):
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    # rotating the scalars by one rank gives something else
+    rotated = scalars[1:] + scalars[:1]
+    assert not np.array_equal(orc.all_reduce(dtype, orc.PREMULSUM, g, sends, scalar=rotated)[0].view(np.uint8),
+                              want.view(np.uint8))
+
+
+def test_premulsum_per_rank_scalars_integers_reduce_scatter_and_reduce():
+    n, C, chunk, align, count = 3, 2, 64, 16, 500
+    g = orc.Geom(n, C, chunk, align)
+    ks = [7, -3, 1_000_003]
+    sends = [datagen.make(orc.I32, 1200 + r, count * n) for r in range(n)]
+    exact = np.array([wrap(sum(wrap(int(sends[r][i]) * ks[r], 32, True) for r in range(n)), 32, True)
+                      for i in range(count * n)], np.int32)
+    scalars = [orc.scalar_bits(orc.I32, k) for k in ks]
+    for r, got in enumerate(orc.reduce_scatter(orc.I32, orc.PREMULSUM, g, sends, scalar=scalars)):
+        assert np.array_equal(got, exact[r * count:(r + 1) * count])
+    root = 2
+    assert np.array_equal(orc.reduce(orc.I32, orc.PREMULSUM, g, root, sends, scalar=scalars)[root], exact)
+    for got in orc.all_reduce(orc.I32, orc.PREMULSUM, g, sends, scalar=scalars):
+        assert np.array_equal(got, exact)
+
+
+def test_premulsum_per_rank_scalars_floats_reduce_scatter_and_reduce():
+    n, C, chunk, align, count = 4, 2, 64, 16, 1000
+    g = orc.Geom(n, C, chunk, align)
+    scalars = [orc.scalar_bits(orc.F32, v) for v in (0.3, -1.7, 2.5, 0.01)]
+    sends = [datagen.make(orc.F32, 1300 + r, count * n) for r in range(n)]
+    scaled = [np_mul(orc.F32, sends[r], scalars[r]) for r in range(n)]
+    for d, got in enumerate(orc.reduce_scatter(orc.F32, orc.PREMULSUM, g, sends, scalar=scalars)):
+        blocks = [x[d * count:(d + 1) * count] for x in scaled]
+        acc = blocks[(d + 1) % n]
+        for j in range(2, n + 1):
+            acc = blocks[(d + j) % n] + acc
+        assert np.array_equal(got, acc)
+    root = 1
+    acc = scaled[(root + 1) % n]
+    for j in range(2, n + 1):
+        acc = scaled[(root + j) % n] + acc
+    assert np.array_equal(orc.reduce(orc.F32, orc.PREMULSUM, g, root, sends, scalar=scalars)[root], acc)
+
+
 # ---- Max / Min with NaN operands: fmaxf / fminf return the operand that is a number -------------------------
 # (src/include/reduce_kernel.h:442-469; fp16 goes through float, :344-362,393-411).  A NaN comes out only where
 # every operand is a NaN.  Which of two zeros of different sign comes out is not fixed by fmax / fmin and stays
