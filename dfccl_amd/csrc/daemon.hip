@@ -232,6 +232,20 @@ __device__ __forceinline__ void storeStruct(T* dst, const T& src) {
   for (unsigned i = 0; i < sizeof(T) / 8; i++) d[i] = s[i];
 }
 
+// The value lane `srcLane` of the wave holds (srcLane is the same in every lane): a register read, no LDS.
+__device__ __forceinline__ uint64_t readLane64(uint64_t v, int srcLane) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, srcLane);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), srcLane);
+  return (uint64_t)lo | ((uint64_t)hi << 32);
+}
+
+// A 64-bit value that is the same in every lane, into scalar registers (the first lane's copy).
+__device__ __forceinline__ uint64_t uniform64(uint64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (uint64_t)lo | ((uint64_t)hi << 32);
+}
+
 __device__ __forceinline__ uint64_t waveMin64(uint64_t v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
@@ -473,7 +487,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
     if (polls > 1) st.idle += polls - 1;  // (the same count in every lane: the loop ends on a ballot)
   }
   const bool valid = lane < nlanes && (w & ~kPtrMask) == tagWant;
-  const uint64_t ctrlWord = __shfl(w, 60);
+  const uint64_t ctrlWord = readLane64(w, 60);  // (into scalar registers: the wave branches on it)
   const uint32_t ctrl = (uint32_t)ctrlWord, statsReq = (uint32_t)(ctrlWord >> 32);
   if (statsReq != st.statsReqSeen) {
     st.statsReqSeen = statsReq;
@@ -523,7 +537,7 @@ __device__ __forceinline__ void pollHost(const DaemonArgs& A, const RankDev& R, 
     if (R.nChannels > 1) {
       f = ~0ull;
       if (lane < R.nChannels) f = __hip_atomic_load(G(&R.wgFrontier[lane]), __ATOMIC_RELAXED, DFCCL_AGENT);
-      f = waveMin64(f);
+      f = uniform64(waveMin64(f));
     }
     if (f != published) {
       if (lane == 0) __hip_atomic_store(G(R.sqHead), f, __ATOMIC_RELAXED, DFCCL_SYSTEM);
@@ -761,19 +775,6 @@ __device__ __forceinline__ void moveSliceScaled(int dtype, const void* s0, const
 }
 
 // Direct protocol data movement.  A "tile" is one rank's chunk of one loop.
-
-// The value lane `srcLane` of the wave holds (srcLane is the same in every lane): a register read, no LDS.
-__device__ __forceinline__ uint64_t readLane64(uint64_t v, int srcLane) {
-  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, srcLane);
-  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), srcLane);
-  return (uint64_t)lo | ((uint64_t)hi << 32);
-}
-
-__device__ __forceinline__ uint64_t uniform64(uint64_t v) {
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-  return (uint64_t)lo | ((uint64_t)hi << 32);
-}
 
 // dst[k][off..] = src[0][off..] (op) src[1][off..] ... (op) src[n-1][off..] for every k < nd, folded left to
 // right with every step rounded to the storage type: with src = in[c+1], in[c+2], ..., in[c] this is the ring's

@@ -1015,12 +1015,10 @@ DFCCL_API ncclResult_t ofcclFinalizeRankCtx7StartHostThrds(ofcclRankCtx_t c) {
     p.scalePtr = (const void*)(uintptr_t)g->scalePtr[(size_t)rank];
     if (g->proto == kProtoDirect && g->scaleKind == kScalePre && p.scalePtr == nullptr) {
       // the peers fold this rank's input: they find its scalar next to its buffer pointers.  Only the `scale`
-      // words of this rank's row are written (nothing has been announced through them yet).
-      std::vector<PeerPub> row((size_t)g->nChannels);
-      memset(row.data(), 0, row.size() * sizeof(PeerPub));
-      for (auto& e : row) e.scale = p.scaleBits;
-      HIPCHECK(hipMemcpy(g->pubs + (size_t)rank * g->nChannels, row.data(), row.size() * sizeof(PeerPub),
-                         hipMemcpyHostToDevice));
+      // word of every channel of this rank's row is written (the tagged words beside it belong to the kernel).
+      for (int ch = 0; ch < g->nChannels; ch++)
+        HIPCHECK(hipMemcpy(&g->pubs[(size_t)rank * g->nChannels + ch].scale, &p.scaleBits, sizeof(p.scaleBits),
+                           hipMemcpyHostToDevice));
     }
     p.loopsPerInstance = g->loopsPerInstance;
     p.lastChunkElems = g->lastChunkElems;
