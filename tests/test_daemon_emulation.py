@@ -190,7 +190,7 @@ def test_parity_tests_on_the_emulation(stress):
               "EMUL_JITTER": "30", "EMUL_WATCHDOG_S": "120"})
     pick = ("test_small_all_reduce_and_in_place or test_in_place_and_absent_buffers or golden or "
             "test_other_collectives_disordered or test_rank_by_rank or forced_preemption or avg_small_and_ragged or "
-            "premul_sum or nan_operands")
+            "premul_sum or nan_operands or empty_collectives")
     r = subprocess.run([sys.executable, "-m", "pytest", os.path.join(HERE, "test_daemon_gpu.py"),
                         os.path.join(HERE, "test_golden.py"), "-q", "-m", "gpu", "-x", "-p", "no:cacheprovider",
                         "--timeout", "600", "-k", pick], env=e, capture_output=True, text=True, timeout=1200,

@@ -834,3 +834,29 @@ def test_small_all_reduce_repeated_and_fallbacks(knobs, monkeypatch):
                 assert np.array_equal(to_np(dtype, recvs[r]), want[r]), (rep, r)
         stats = ring.stats()
         assert stats["cqesWritten"] == 40 * n
+
+
+def test_empty_collectives_complete_and_touch_nothing():
+    # count 0 (NCCL accepts it: nothing moves): every kind completes with a callback, twice in a row, and the
+    # one-element buffers that are passed keep their contents; a real collective registered beside them still works
+    from dfccl_amd.ring import VirtualRing
+    n = 3
+    with VirtualRing(n) as ring:
+        for cid, kind in enumerate(("all_reduce", "reduce_scatter", "all_gather", "reduce", "broadcast")):
+            ring.prepare(cid, kind, 0, orc.F32, orc.SUM, root=1)
+        ring.prepare(5, "all_reduce", 1000, orc.I32, orc.SUM)
+        ring.finalize()
+        marks = [torch.full((4,), 7.0, device=gpu_util.DEVICE) for _ in range(n)]
+        outs = [torch.full((4,), 9.0, device=gpu_util.DEVICE) for _ in range(n)]
+        sends_np, sends, recvs = make_buffers("all_reduce", orc.I32, n, 1000, 2500)
+        torch.cuda.current_stream().synchronize()
+        for rep in range(2):
+            for r in range(n):
+                for cid in range(5):
+                    ring.submit(r, cid, marks[r], outs[r])
+                ring.submit(r, 5, sends[r], recvs[r])
+            ring.wait([(r, cid) for r in range(n) for cid in range(6)], timeout=30)
+        want = orc.all_reduce(orc.I32, orc.SUM, geom_of(ring, 5), sends_np)
+        for r in range(n):
+            assert bool((marks[r] == 7.0).all()) and bool((outs[r] == 9.0).all()), r
+            assert np.array_equal(to_np(orc.I32, recvs[r]), want[r]), r
