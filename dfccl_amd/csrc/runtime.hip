@@ -542,11 +542,12 @@ static void planGroup(CommGroup* g) {
     sliceBytes = stepBytes;
     g->slicesPerChunk = 1;
     g->fifoSlots = 8;
-  } else {  // CHUNKSTEPS 4, SLICESTEPS 2
+  } else {  // CHUNKSTEPS 4, SLICESTEPS 2: NCCL_STEPS / SLICESTEPS = 4 slices of a link in flight
     chunkBytes = stepBytes * 4;
     sliceBytes = stepBytes * 2;
     g->slicesPerChunk = 2;
-    g->fifoSlots = 4;
+    // (DFCCL_FIFO_SLOTS: more slots than the reference's four give neighbours more slack, at that much more memory)
+    g->fifoSlots = (int)std::min<int64_t>(16, std::max<int64_t>(2, envInt("DFCCL_FIFO_SLOTS", 4)));
   }
   // Default: share the workgroups the GPU keeps resident (one per CU) among the ranks that will run together,
   // which is the larger of this communicator's size and the rank contexts created on the device so far, and

@@ -83,6 +83,9 @@ SCENARIOS = [
     ("mixed-direct-tiny-budget", TINY, ["mixed", "4", "2"]),
     ("mixed-fifo", {"DFCCL_PROTO": "fifo"}, ["mixed", "3", "2"]),
     ("mixed-fifo-tiny-budget", dict(TINY, DFCCL_PROTO="fifo"), ["mixed", "3", "2"]),
+    # FIFO links of two and of eight slices instead of the reference's four
+    ("mixed-fifo-2-slots", {"DFCCL_PROTO": "fifo", "DFCCL_FIFO_SLOTS": "2"}, ["mixed", "3", "1"]),
+    ("mixed-fifo-8-slots", {"DFCCL_PROTO": "fifo", "DFCCL_FIFO_SLOTS": "8"}, ["mixed", "3", "1"]),
     # forced preemption after every slice / tile
     ("forced-direct", {"DFCCL_FORCE_QUIT_EVERY": "1"}, ["repeat", "2", "40000", "2", "1"]),
     ("forced-fifo", {"DFCCL_FORCE_QUIT_EVERY": "2", "DFCCL_PROTO": "fifo"}, ["repeat", "3", "40000", "2", "1"]),
