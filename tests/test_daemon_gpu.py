@@ -236,6 +236,37 @@ def test_premul_sum_scalar_in_device_memory(dtype):
                 assert np.array_equal(to_np(dtype, rs_recv[r]), want[r]), r
 
 
+def test_premul_sum_ranks_mix_host_and_device_scalars():
+    # even ranks give their scalar by value, odd ranks leave it in device memory
+    import dfccl_amd
+    from dfccl_amd import api
+    from dfccl_amd.ring import VirtualRing
+    dtype, n, count = orc.F32, 4, 20011
+    values = PREMUL_VALUES[dtype][:n]
+    slots = torch.zeros(n * 4, dtype=torch.float32, device=gpu_util.DEVICE)
+    slots.copy_(torch.tensor([v for v in values for _ in range(4)], dtype=torch.float32))
+    torch.cuda.current_stream().synchronize()
+    with VirtualRing(n) as ring:
+        comms = api.VirtualComm.create_all(n)
+        for r, ctx in enumerate(ring.ctxs):
+            if r % 2 == 0:
+                op = comms[r].create_premul_sum(dtype, scalar_bytes_of(dtype, values[r]))
+            else:
+                op = comms[r].create_premul_sum(dtype, device_ptr=slots.data_ptr() + 16 * r)
+            ctx.prepare_all_reduce(count, dtype, op, comms[r], 0)
+            ring.done[(r, 0)] = threading.Event()
+        ring.comms[0] = comms
+        ring.kinds[0] = "all_reduce"
+        ring.finalize()
+        sends_np, sends, recvs = make_buffers("all_reduce", dtype, n, count, 298)
+        want = orc.all_reduce(dtype, orc.PREMULSUM, geom_of(ring, 0), sends_np,
+                              scalar=[orc.scalar_bits(dtype, v) for v in values])
+        for rep in range(2):
+            ring.run(0, sends, recvs, timeout=30)
+            for r in range(n):
+                assert np.array_equal(to_np(dtype, recvs[r]), want[r]), (rep, r)
+
+
 def test_premul_sum_on_a_communicator_of_one_rank():
     # a sum of one term is still multiplied, out of place and in place
     from dfccl_amd.ring import VirtualRing
