@@ -177,14 +177,15 @@ def test_premul_sum_operator(dtype, per_rank):
         assert np.array_equal(to_np(dtype, rd_recv[root]), want[root])
 
 
-@pytest.mark.parametrize("n,count", [(2, 1000), (8, 4099), (3, 200003)])
+@pytest.mark.parametrize("n,count", [(2, 1000), (8, 4099), (3, 200003), (10, 5003)])
 def test_premul_sum_scalar_per_rank_small_and_large(n, count):
-    # sizes that wave 0 folds alone (2 and 8 ranks) and one that takes several channels
+    # sizes that wave 0 folds alone (2 and 8 ranks), one that takes several channels, and more ranks than the direct
+    # protocol folds in one pass (the FIFO ring then, whatever protocol was asked for)
     from dfccl_amd.ring import VirtualRing
     if gpu_util.EMULATED:
         count = min(count, 40003)
     for dtype in (orc.F16, orc.I64):
-        values = PREMUL_VALUES[dtype][:n]
+        values = [PREMUL_VALUES[dtype][r % 8] * (1 + r // 8) for r in range(n)]
         bits = [orc.scalar_bits(dtype, v) for v in values]
         with VirtualRing(n) as ring:
             ring.prepare(0, "all_reduce", count, dtype, premul=[scalar_bytes_of(dtype, v) for v in values])
